@@ -1,0 +1,69 @@
+"""ctypes binding of libbhi_hip.so (the C ABI declared in include/bhi.h).
+
+The library is built in-tree by ``python -m bf16_huffman_infer_amd.csrc.build``.  There
+is no fallback: if it is missing every op of this package raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libbhi_hip.so")
+
+_vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+
+_SIGNATURES = {
+    "bhi_constants": (_i32, [ctypes.POINTER(ctypes.c_int32), _i32]),
+    "bhi_chunks_per_group": (_i32, [_i32, _i32, _i32]),
+    "bhi_last_error_string": (ctypes.c_char_p, []),
+    "bhi_gemv_bf16_huffman": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,
+                                     _i32, _i32, _i32, _i32, _vp]),
+    "bhi_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,
+                                  _i32, _i32, _i32, _vp]),
+    "bhi_huffman_encode": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp]),
+    "bhi_encode_capacity": (_i64, [_i32]),
+    "bhi_gemv_bf16_ans": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
+    "bhi_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "bhi_ans_encode": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp]),
+    "bhi_ans_encode_capacity": (_i64, [_i32]),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Returns the loaded library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build the HIP extension first "
+                "(python -m bf16_huffman_infer_amd.csrc.build). There is no CPU fallback.")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().bhi_last_error_string().decode()
+        raise RuntimeError(f"{what} failed (code {rc}): {msg}")
+
+
+_CONST_NAMES = (
+    "format_version", "lanes", "group_rows", "step_cols", "table_bits", "init_words",
+    "header_bits", "max_batch", "ans_precision", "align_words", "tail_pad_words",
+    "target_tasks", "max_task_steps",
+)
+
+
+def constants() -> dict:
+    lib = load()
+    buf = (ctypes.c_int32 * len(_CONST_NAMES))()
+    n = lib.bhi_constants(buf, len(_CONST_NAMES))
+    assert n == len(_CONST_NAMES), "constant table of the library and of the binding differ"
+    return dict(zip(_CONST_NAMES, buf))

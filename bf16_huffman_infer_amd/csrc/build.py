@@ -1,0 +1,34 @@
+"""Builds libbhi_hip.so for gfx950 next to the package (python -m bf16_huffman_infer_amd.csrc.build)."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(HERE)
+SOURCES = ["bhi_api.hip", "bhi_huffman.hip", "bhi_ans.hip"]
+LIB = os.path.join(PKG, "libbhi_hip.so")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-variable",
+]
+
+
+def build(verbose: bool = True) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *FLAGS, *[os.path.join(HERE, s) for s in SOURCES], "-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    out = "\n".join(l for l in (proc.stdout + proc.stderr).splitlines()
+                    if "packed-fp32-ops" not in l)
+    if verbose and out.strip():
+        print(out)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,375 @@
+"""Compressed-weight modules, conversion and the ``F.linear`` dispatch.
+
+Public surface of the reference's ``bf16_huffman_infer/functional.py``:
+``HuffmanWeight``, ``ANSWeight``, ``CompressedLinear``, ``convert``,
+``convert_all_linear``, ``linear_huffman`` (plus ``linear_ans``, ``mv_huffman``,
+``mv_ans``).  Module buffers keep the reference's names and dtypes
+(``rem, exp, offsets, LUT1..LUT4, code_lengths`` / ``rem, exp, offsets, LUT``), the
+bytes inside ``rem``/``exp``/``offsets``/``LUT1`` follow the wave64 layout of this
+package's HIP kernels.
+"""
+from typing import Optional
+
+import torch
+from torch import Tensor, nn
+import torch.nn.functional as F
+from tqdm import tqdm
+
+from . import _lib
+from .ans import RANSEncoder
+from .huffman import LUTHuffmanEncoder
+from .ops import (ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemv_bf16_ans,
+                  gemv_bf16_huffman, huffman_decode, huffman_encode)
+from .utils import get_block_size_n, split_bf16
+
+ANS_PRECISION = 8
+MAX_FUSED_BATCH = 8
+GROUP_ROWS = 4
+STEP_COLS = 128
+LANES = 64
+LANE_COLS = 8
+ENCODE_PART_BYTES = 256 << 20       # scratch bound per encode call
+
+__all__ = [
+    "linear_huffman",
+    "linear_ans",
+    "HuffmanWeight",
+    "ANSWeight",
+    "CompressedLinear",
+    "convert_all_linear",
+    "convert",
+]
+
+
+def _lane_order(plane: Tensor, split_k: int) -> Tensor:
+    """[M, K] byte plane -> [split_k, G, S, 64, 8]: (split, row group, step, lane, column)."""
+    M, K = plane.shape
+    Ks = K // split_k
+    G, S = M // GROUP_ROWS, Ks // STEP_COLS
+    x = plane.view(G, GROUP_ROWS, split_k, S, STEP_COLS // LANE_COLS, LANE_COLS)     # g i k t b j
+    return x.permute(2, 0, 3, 4, 1, 5).reshape(split_k, G, S, LANES, LANE_COLS)
+
+
+def _check_weight_call(A_rem: Tensor, A_exp: Tensor, X: Tensor):
+    split_k, M, N = A_rem.shape
+    assert M % 128 == 0
+    assert N % 128 == 0
+    assert X.dim() == 3 and X.size(-1) == N
+    assert X.dtype == torch.bfloat16
+    assert A_rem.device.type == A_exp.device.type == X.device.type == 'cuda'
+    assert A_rem.device == A_exp.device == X.device
+
+
+def mv_huffman(
+    A_rem: Tensor, A_exp: Tensor, X: Tensor,
+    offsets: Tensor,
+    LUT1: Tensor, LUT2: Tensor, LUT3: Tensor, LUT4: Tensor,
+    code_lengths: Tensor,
+) -> Tensor:
+    """Y[b, :] = W @ X[b, :] for b < 8 with W held compressed (reference ``functional.py:28-63``)."""
+    split_k, M, N = A_rem.shape
+    X = X.view(-1, split_k, N)
+    _check_weight_call(A_rem, A_exp, X)
+    Y = torch.empty((X.size(0), M), dtype=torch.bfloat16, device=A_rem.device)
+    gemv_bf16_huffman(A_rem.contiguous(), A_exp.contiguous(), X.contiguous(), Y, offsets.contiguous(),
+                      LUT1.contiguous(), LUT2.contiguous(), LUT3.contiguous(), LUT4.contiguous(),
+                      code_lengths.contiguous())
+    return Y
+
+
+def mv_ans(A_rem: Tensor, A_exp: Tensor, X: Tensor, offsets: Tensor, LUT: Tensor) -> Tensor:
+    """rANS counterpart of :func:`mv_huffman` (reference ``functional.py:414-444``)."""
+    split_k, M, N = A_rem.shape
+    X = X.view(-1, split_k, N)
+    _check_weight_call(A_rem, A_exp, X)
+    Y = torch.empty((X.size(0), M), dtype=torch.bfloat16, device=A_rem.device)
+    gemv_bf16_ans(A_rem.contiguous(), A_exp.contiguous(), X.contiguous(), Y, offsets.contiguous(), LUT.contiguous())
+    return Y
+
+
+class HuffmanWeight(nn.Module):
+    """A BF16 weight ``[M, K]`` stored as a raw sign/mantissa plane plus a Huffman-coded
+    exponent stream.  Passing the module as the weight of ``F.linear`` runs the fused
+    kernels (reference ``functional.py:66-242``)."""
+
+    def __init__(
+        self,
+        rem: Tensor,
+        exp: Tensor,
+        offsets: Tensor,
+        LUT1: Tensor,
+        LUT2: Tensor,
+        LUT3: Tensor,
+        LUT4: Tensor,
+        code_lengths: Tensor,
+    ):
+        super().__init__()
+        self.rem = nn.Buffer(rem)
+        self.exp = nn.Buffer(exp)
+        self.offsets = nn.Buffer(offsets)
+        self.LUT1 = nn.Buffer(LUT1)
+        self.LUT2 = nn.Buffer(LUT2)
+        self.LUT3 = nn.Buffer(LUT3)
+        self.LUT4 = nn.Buffer(LUT4)
+        self.code_lengths = nn.Buffer(code_lengths)
+
+    def kwargs(self) -> dict[str, Tensor]:
+        return dict(self.named_buffers())
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        if func is not F.linear:
+            return NotImplemented
+        return linear_huffman(*args, **(kwargs or {}))
+
+    def _empty_weight(self) -> Tensor:
+        split_k, M, Ks = self.rem.shape
+        assert self.rem.device.type == 'cuda'
+        return torch.empty((M, split_k * Ks), dtype=torch.bfloat16, device=self.rem.device)
+
+    def get_weight(self) -> Tensor:
+        """The original BF16 weight, bit for bit."""
+        weight = self._empty_weight()
+        huffman_decode(self.rem, self.exp, weight, self.offsets,
+                       self.LUT1, self.LUT2, self.LUT3, self.LUT4, self.code_lengths)
+        return weight
+
+    # ------------------------------------------------------------------ compression
+    @classmethod
+    def get_codec(cls, a: Tensor) -> LUTHuffmanEncoder:
+        """One code per weight matrix, built from the histogram of exponent pairs."""
+        device = torch.device('cuda', 0)
+        _, exp = split_bf16(a.detach().to(device))
+        pairs = exp[:, 0::2].to(torch.int32) | (exp[:, 1::2].to(torch.int32) << 8)
+        counts = torch.bincount(pairs.flatten(), minlength=65536)
+        codec = LUTHuffmanEncoder()
+        codec.build_lut(counts.cpu())
+        return codec
+
+    @classmethod
+    def get_lut_kwargs(cls, codec: LUTHuffmanEncoder) -> dict[str, Tensor]:
+        return {
+            'LUT1': torch.from_numpy(codec.LUT1.copy()),
+            'LUT2': torch.from_numpy(codec.LUT2.copy()),
+            'LUT3': torch.from_numpy(codec.LUT3.copy()),
+            'LUT4': torch.from_numpy(codec.LUT4.copy()),
+            'code_lengths': torch.from_numpy(codec.code_lengths.copy()),
+        }
+
+    @classmethod
+    def capacity(cls, n_steps: int) -> int:
+        return encode_capacity(n_steps)
+
+    @classmethod
+    def compress_groups(cls, x: Tensor, codec) -> tuple[Tensor, Tensor]:
+        """x: uint8 ``[tasks, steps*512]`` lane-ordered exponents of equally long tasks ->
+        (streams int32 ``[tasks, capacity]``, words used per task)."""
+        device = x.device
+        n_steps = x.size(1) // (LANES * LANE_COLS)
+        out = torch.zeros(x.size(0), cls.capacity(n_steps), dtype=torch.int32, device=device)
+        lengths = torch.zeros(x.size(0), dtype=torch.int32, device=device)
+        table = torch.from_numpy(codec.enc_table.view('int32').copy()).to(device)
+        huffman_encode(x, table, out, lengths)
+        return out, lengths
+
+    @classmethod
+    def compress_split_n(cls, a: Tensor, n: int = 2):
+        """Compress ``a`` with ``n`` column splits (the reference's ``compress_split_n``,
+        ``functional.py:195-238``)."""
+        assert a.dim() == 2 and a.dtype == torch.bfloat16
+        a = a.detach()
+        M, K = a.shape
+        assert M % 128 == 0 and K % n == 0 and (K // n) % STEP_COLS == 0, a.shape
+        Ks = K // n
+        S, G = Ks // STEP_COLS, M // GROUP_ROWS
+        device = torch.device('cuda', 0)
+        lib = _lib.load()
+        consts = _lib.constants()
+        nc = lib.bhi_chunks_per_group(M, Ks, n)
+
+        codec = cls.get_codec(a)
+        rem, exp = split_bf16(a.to(device))
+        rem = _lane_order(rem, n).reshape(n, M, Ks).contiguous()
+        sym = _lane_order(exp, n)                                           # [n, G, S, 64, 8]
+        del exp
+
+        lengths = torch.zeros(n, G, nc, dtype=torch.int64, device=device)
+        pieces = []                                                          # (chunk, first task, streams, lengths)
+        for c in range(nc):
+            t0, t1 = (S * c) // nc, (S * (c + 1)) // nc
+            tasks = sym[:, :, t0:t1].reshape(n * G, (t1 - t0) * LANES * LANE_COLS)
+            per_call = max(1, ENCODE_PART_BYTES // (4 * cls.capacity(t1 - t0)))
+            for first in range(0, n * G, per_call):
+                out, ln = cls.compress_groups(tasks[first:first + per_call].contiguous(), codec)
+                used = int(ln.max().item())
+                pieces.append((c, first, out[:, :used].clone(), ln.to(torch.int64)))
+                lengths.view(n * G, nc)[first:first + ln.numel(), c] = ln
+        del sym
+
+        total = int(lengths.sum().item())
+        assert total + consts['tail_pad_words'] < 2 ** 31, "exponent stream too large for int32 offsets"
+        starts = (torch.cumsum(lengths.flatten(), 0) - lengths.flatten()).view(n * G, nc)
+        words = torch.zeros(total + consts['tail_pad_words'], dtype=torch.int32, device=device)
+        for c, first, out, ln in pieces:
+            cols = torch.arange(out.size(1), device=device)[None, :]
+            keep = cols < ln[:, None]
+            dest = (starts[first:first + ln.numel(), c][:, None] + cols)[keep]
+            words[dest] = out[keep]
+        offsets = torch.zeros(n, G, GROUP_ROWS, dtype=torch.int32, device=device)
+        offsets[:, :, :nc] = starts.view(n, G, nc).to(torch.int32)
+
+        return cls(
+            rem=rem.cpu(),
+            exp=words.cpu(),
+            offsets=offsets.view(n, M).cpu(),
+            **cls.get_lut_kwargs(codec),
+        )
+
+    @classmethod
+    def compress(cls, a: Tensor):
+        return cls.compress_split_n(a, n=get_block_size_n(a)[0])
+
+
+class ANSWeight(HuffmanWeight):
+    """Same planes and stream layout with an interleaved rANS exponent stream
+    (reference ``functional.py:245-310``)."""
+
+    def __init__(self, rem: Tensor, exp: Tensor, offsets: Tensor, LUT: Tensor):
+        nn.Module.__init__(self)
+        self.rem = nn.Buffer(rem)
+        self.exp = nn.Buffer(exp)
+        self.offsets = nn.Buffer(offsets)
+        self.LUT = nn.Buffer(torch.as_tensor(LUT))
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        if func is not F.linear:
+            return NotImplemented
+        return linear_ans(*args, **(kwargs or {}))
+
+    def get_weight(self) -> Tensor:
+        weight = self._empty_weight()
+        ans_decode(self.rem, self.exp, weight, self.offsets, self.LUT)
+        return weight
+
+    @classmethod
+    def get_codec(cls, a: Tensor) -> RANSEncoder:
+        device = torch.device('cuda', 0)
+        _, exp = split_bf16(a.detach().to(device))
+        counts = torch.bincount(exp.flatten().to(torch.int32), minlength=256)
+        return RANSEncoder(counts.tolist(), precision=ANS_PRECISION)
+
+    @classmethod
+    def get_lut_kwargs(cls, codec: RANSEncoder) -> dict[str, Tensor]:
+        lut = torch.tensor(codec.decode_lut, dtype=torch.int32)
+        return {'LUT': (lut[:, 0] << 24) | (lut[:, 1] << 12) | lut[:, 2]}
+
+    @classmethod
+    def capacity(cls, n_steps: int) -> int:
+        return ans_encode_capacity(n_steps)
+
+    @classmethod
+    def compress_groups(cls, x: Tensor, codec: RANSEncoder) -> tuple[Tensor, Tensor]:
+        device = x.device
+        n_steps = x.size(1) // (LANES * LANE_COLS)
+        out = torch.zeros(x.size(0), cls.capacity(n_steps), dtype=torch.int32, device=device)
+        lengths = torch.zeros(x.size(0), dtype=torch.int32, device=device)
+        freq = torch.tensor(codec.freq, dtype=torch.int32, device=device)
+        cum = torch.tensor(codec.cum, dtype=torch.int32, device=device)
+        ans_encode(x, freq, cum, out, lengths)
+        return out, lengths
+
+
+class CompressedLinear(nn.Module):
+    def __init__(self, weight: HuffmanWeight, bias: Optional[Tensor]) -> None:
+        super().__init__()
+        self.weight = weight
+        self.bias = bias
+
+    def forward(self, input: Tensor) -> Tensor:
+        return F.linear(input, self.weight, self.bias)
+
+
+def _weight_bytes(w: nn.Module) -> int:
+    return sum(b.nelement() * b.element_size() for b in w.buffers())
+
+
+def convert(linear: nn.Linear, name, disable_precision_check=True, algo='huffman') -> nn.Module:
+    """Compress one ``nn.Linear`` (reference ``functional.py:323-375``).
+
+    Returns the original module when compression does not shrink it or when the decoded
+    weight is not bit-identical; with ``disable_precision_check=False`` also when one
+    random GEMV deviates by 2 % or more from the dense layer.
+    """
+    assert algo in ('huffman', 'ans', 'smallest')
+    if algo == 'huffman':
+        weight = HuffmanWeight.compress(linear.weight)
+    elif algo == 'ans':
+        weight = ANSWeight.compress(linear.weight)
+    else:
+        weight = min([HuffmanWeight.compress(linear.weight), ANSWeight.compress(linear.weight)], key=_weight_bytes)
+
+    module = CompressedLinear(weight=weight, bias=linear.bias)
+    ori_size = linear.weight.nelement() * linear.weight.element_size()
+    ratio = _weight_bytes(module.weight) / ori_size
+
+    linear.cuda()
+    module.cuda()
+    x = torch.randn(1, linear.in_features, dtype=torch.bfloat16, device='cuda')
+    with torch.no_grad():
+        y1 = linear(x)
+        y2 = module(x)
+        lossless = torch.equal(module.weight.get_weight().view(torch.int16), linear.weight.view(torch.int16))
+    max_rtol = ((y2 - y1).abs() / y1.abs().clamp(min=1e-4)).max().item()
+    linear.cpu()
+    module.cpu()
+
+    fallback = False
+    if ratio >= 1:
+        print(f'\nWarning! {name} ratio = {ratio:.2%}')
+        fallback = True
+    if not lossless:
+        print(f'\nWarning! {name} does not decode to the original weight')
+        fallback = True
+    if not disable_precision_check and max_rtol >= 0.02:
+        print(f'\nWarning! {name} output mismatch: max rtol = {max_rtol:.2f}')
+        fallback = True
+    if fallback:
+        print('Fallback to regular nn.Linear')
+        return linear
+    return module
+
+
+def convert_all_linear(model: nn.Module, min_out_features=4096, progress=True, algo='huffman') -> None:
+    """Replace every ``nn.Linear`` with at least ``min_out_features`` outputs in place."""
+    targets = [name for name, m in model.named_modules()
+               if isinstance(m, nn.Linear) and m.out_features >= min_out_features]
+    for name in tqdm(targets, disable=not progress):
+        model.set_submodule(name, convert(model.get_submodule(name), name, algo=algo))
+
+
+def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tensor], fused) -> Tensor:
+    assert input.dim() >= 2, input
+    shape = input.shape
+    input = input.flatten(0, -2)
+    if input.size(0) <= MAX_FUSED_BATCH:
+        output = fused(input)
+        if bias is not None:
+            output += bias[None, :]
+    else:
+        output = F.linear(input, weight.get_weight(), bias)
+    return output.unflatten(0, shape[:-1])
+
+
+def linear_huffman(input: Tensor, weight: HuffmanWeight, bias: Optional[Tensor] = None) -> Tensor:
+    """``F.linear`` with a :class:`HuffmanWeight`: fused kernel up to 8 rows, else decode +
+    dense GEMM (reference ``functional.py:390-411``)."""
+    return _linear_compressed(input, weight, bias, lambda x: mv_huffman(
+        weight.rem, weight.exp, x, weight.offsets,
+        weight.LUT1, weight.LUT2, weight.LUT3, weight.LUT4, weight.code_lengths))
+
+
+def linear_ans(input: Tensor, weight: ANSWeight, bias: Optional[Tensor] = None) -> Tensor:
+    """rANS counterpart of :func:`linear_huffman` (reference ``functional.py:447-466``)."""
+    return _linear_compressed(input, weight, bias, lambda x: mv_ans(
+        weight.rem, weight.exp, x, weight.offsets, weight.LUT))

@@ -1,0 +1,207 @@
+"""The six custom ops of namespace ``bf16_huffman_infer`` on HIP.
+
+Same op names, schemas and positional wrappers as the reference
+(``bf16_huffman_infer/src/bf16_huffman_infer.cpp:29-35``, ``ops.py:6-61``).  The schemas
+are registered from Python and the ``CUDA`` dispatch key (the key ROCm devices use)
+forwards raw device pointers and the current torch stream to ``libbhi_hip.so``.
+No other key is registered: CPU tensors are rejected by the dispatcher, as the
+reference rejects them with asserts.
+
+Every op mutates caller-allocated outputs and returns nothing; nothing here
+synchronises or allocates, so the ops can be captured in a HIP graph.
+"""
+import torch
+from torch import Tensor
+
+from . import _lib
+
+_LIB = torch.library.Library("bf16_huffman_infer", "DEF")
+_LIB.define("gemv_bf16_huffman(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, "
+            "Tensor LUT1, Tensor LUT2, Tensor LUT3, Tensor LUT4, Tensor code_lengths) -> ()")
+_LIB.define("huffman_encode(Tensor data, Tensor LUT, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
+_LIB.define("huffman_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, "
+            "Tensor LUT1, Tensor LUT2, Tensor LUT3, Tensor LUT4, Tensor code_lengths) -> ()")
+_LIB.define("gemv_bf16_ans(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
+_LIB.define("ans_encode(Tensor data, Tensor freq, Tensor cum, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
+_LIB.define("ans_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
+
+LANE_BYTES_PER_STEP = 512          # 64 lanes x 8 exponent bytes
+
+
+def _stream(t: Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _req(t: Tensor, dtype, name: str, ref: Tensor = None) -> int:
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name}: must be contiguous")
+    if ref is not None and t.device != ref.device:
+        raise RuntimeError(f"{name}: on {t.device}, expected {ref.device}")
+    return t.data_ptr()
+
+
+def _weight_dims(A_rem: Tensor, offsets: Tensor):
+    if A_rem.dim() != 3:
+        raise RuntimeError(f"A_rem must be [split_k, M, Ks], got {tuple(A_rem.shape)}")
+    split_k, M, Ks = A_rem.shape
+    if tuple(offsets.shape) != (split_k, M):
+        raise RuntimeError(f"offsets must be [{split_k}, {M}], got {tuple(offsets.shape)}")
+    return split_k, M, Ks
+
+
+def _gemv_common(A_rem, A_exp, X, Y, offsets):
+    split_k, M, Ks = _weight_dims(A_rem, offsets)
+    if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
+        raise RuntimeError(f"X must be [batch, {split_k}, {Ks}], got {tuple(X.shape)}")
+    batch = X.shape[0]
+    if tuple(Y.shape) != (batch, M):
+        raise RuntimeError(f"Y must be [{batch}, {M}], got {tuple(Y.shape)}")
+    return split_k, M, Ks, batch
+
+
+def _gemv_bf16_huffman(A_rem, A_exp, X, Y, offsets, LUT1, LUT2, LUT3, LUT4, code_lengths):
+    lib = _lib.load()
+    split_k, M, Ks, batch = _gemv_common(A_rem, A_exp, X, Y, offsets)
+    with torch.cuda.device(A_rem.device):
+        rc = lib.bhi_gemv_bf16_huffman(
+            _req(A_rem, torch.uint8, "A_rem"), _req(A_exp, torch.int32, "A_exp", A_rem), A_exp.numel(),
+            _req(X, torch.bfloat16, "X", A_rem), _req(Y, torch.bfloat16, "Y", A_rem),
+            _req(offsets, torch.int32, "offsets", A_rem),
+            _req(LUT1, torch.uint8, "LUT1", A_rem), LUT1.numel(),
+            _req(LUT2, torch.uint8, "LUT2", A_rem), _req(LUT3, torch.uint8, "LUT3", A_rem),
+            _req(LUT4, torch.uint8, "LUT4", A_rem), _req(code_lengths, torch.uint8, "code_lengths", A_rem),
+            split_k, M, Ks, batch, _stream(A_rem))
+    _lib.check(rc, "gemv_bf16_huffman")
+
+
+def _huffman_decode(A_rem, A_exp, Y, offsets, LUT1, LUT2, LUT3, LUT4, code_lengths):
+    lib = _lib.load()
+    split_k, M, Ks = _weight_dims(A_rem, offsets)
+    if tuple(Y.shape) != (M, split_k * Ks):
+        raise RuntimeError(f"Y must be [{M}, {split_k * Ks}], got {tuple(Y.shape)}")
+    with torch.cuda.device(A_rem.device):
+        rc = lib.bhi_huffman_decode(
+            _req(A_rem, torch.uint8, "A_rem"), _req(A_exp, torch.int32, "A_exp", A_rem), A_exp.numel(),
+            _req(Y, torch.bfloat16, "Y", A_rem), _req(offsets, torch.int32, "offsets", A_rem),
+            _req(LUT1, torch.uint8, "LUT1", A_rem), LUT1.numel(),
+            _req(LUT2, torch.uint8, "LUT2", A_rem), _req(LUT3, torch.uint8, "LUT3", A_rem),
+            _req(LUT4, torch.uint8, "LUT4", A_rem), _req(code_lengths, torch.uint8, "code_lengths", A_rem),
+            split_k, M, Ks, _stream(A_rem))
+    _lib.check(rc, "huffman_decode")
+
+
+def _encode_dims(data: Tensor, output: Tensor, output_lengths: Tensor):
+    if data.dim() != 2 or data.shape[1] % LANE_BYTES_PER_STEP != 0:
+        raise RuntimeError(f"data must be [tasks, steps*512], got {tuple(data.shape)}")
+    n_tasks, n_steps = data.shape[0], data.shape[1] // LANE_BYTES_PER_STEP
+    if output.dim() != 2 or output.shape[0] != n_tasks or tuple(output_lengths.shape) != (n_tasks,):
+        raise RuntimeError("output must be [tasks, stride] and output_lengths [tasks]")
+    return n_tasks, n_steps
+
+
+def _huffman_encode(data, LUT, output, output_lengths):
+    lib = _lib.load()
+    n_tasks, n_steps = _encode_dims(data, output, output_lengths)
+    if LUT.numel() != 65537:
+        raise RuntimeError("LUT must hold 65537 encoder entries")
+    with torch.cuda.device(data.device):
+        rc = lib.bhi_huffman_encode(
+            _req(data, torch.uint8, "data"), _req(LUT, torch.int32, "LUT", data),
+            _req(output, torch.int32, "output", data), _req(output_lengths, torch.int32, "output_lengths", data),
+            n_tasks, n_steps, output.shape[1], _stream(data))
+    _lib.check(rc, "huffman_encode")
+
+
+def _gemv_bf16_ans(A_rem, A_exp, X, Y, offsets, LUT):
+    lib = _lib.load()
+    split_k, M, Ks, batch = _gemv_common(A_rem, A_exp, X, Y, offsets)
+    if LUT.numel() != 256:
+        raise RuntimeError("LUT must hold 256 rANS slots")
+    with torch.cuda.device(A_rem.device):
+        rc = lib.bhi_gemv_bf16_ans(
+            _req(A_rem, torch.uint8, "A_rem"), _req(A_exp, torch.int32, "A_exp", A_rem), A_exp.numel(),
+            _req(X, torch.bfloat16, "X", A_rem), _req(Y, torch.bfloat16, "Y", A_rem),
+            _req(offsets, torch.int32, "offsets", A_rem), _req(LUT, torch.int32, "LUT", A_rem),
+            split_k, M, Ks, batch, _stream(A_rem))
+    _lib.check(rc, "gemv_bf16_ans")
+
+
+def _ans_decode(A_rem, A_exp, Y, offsets, LUT):
+    lib = _lib.load()
+    split_k, M, Ks = _weight_dims(A_rem, offsets)
+    if tuple(Y.shape) != (M, split_k * Ks):
+        raise RuntimeError(f"Y must be [{M}, {split_k * Ks}], got {tuple(Y.shape)}")
+    if LUT.numel() != 256:
+        raise RuntimeError("LUT must hold 256 rANS slots")
+    with torch.cuda.device(A_rem.device):
+        rc = lib.bhi_ans_decode(
+            _req(A_rem, torch.uint8, "A_rem"), _req(A_exp, torch.int32, "A_exp", A_rem), A_exp.numel(),
+            _req(Y, torch.bfloat16, "Y", A_rem), _req(offsets, torch.int32, "offsets", A_rem),
+            _req(LUT, torch.int32, "LUT", A_rem), split_k, M, Ks, _stream(A_rem))
+    _lib.check(rc, "ans_decode")
+
+
+def _ans_encode(data, freq, cum, output, output_lengths):
+    lib = _lib.load()
+    n_tasks, n_steps = _encode_dims(data, output, output_lengths)
+    if freq.numel() != 256 or cum.numel() != 256:
+        raise RuntimeError("freq and cum must hold 256 entries")
+    with torch.cuda.device(data.device):
+        rc = lib.bhi_ans_encode(
+            _req(data, torch.uint8, "data"), _req(freq, torch.int32, "freq", data), _req(cum, torch.int32, "cum", data),
+            _req(output, torch.int32, "output", data), _req(output_lengths, torch.int32, "output_lengths", data),
+            n_tasks, n_steps, output.shape[1], _stream(data))
+    _lib.check(rc, "ans_encode")
+
+
+for _name, _fn in (("gemv_bf16_huffman", _gemv_bf16_huffman), ("huffman_encode", _huffman_encode),
+                   ("huffman_decode", _huffman_decode), ("gemv_bf16_ans", _gemv_bf16_ans),
+                   ("ans_encode", _ans_encode), ("ans_decode", _ans_decode)):
+    _LIB.impl(_name, _fn, "CUDA")
+
+
+def gemv_bf16_huffman(
+    A_rem: Tensor, A_exp: Tensor, X: Tensor, Y: Tensor,
+    offsets: Tensor,
+    LUT1: Tensor, LUT2: Tensor, LUT3: Tensor, LUT4: Tensor,
+    code_lengths: Tensor,
+) -> None:
+    torch.ops.bf16_huffman_infer.gemv_bf16_huffman.default(
+        A_rem, A_exp, X, Y, offsets, LUT1, LUT2, LUT3, LUT4, code_lengths)
+
+
+def huffman_encode(data: Tensor, LUT: Tensor, output: Tensor, output_lengths: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.huffman_encode.default(data, LUT, output, output_lengths)
+
+
+def huffman_decode(
+    A_rem: Tensor, A_exp: Tensor, Y: Tensor,
+    offsets: Tensor,
+    LUT1: Tensor, LUT2: Tensor, LUT3: Tensor, LUT4: Tensor,
+    code_lengths: Tensor,
+) -> None:
+    torch.ops.bf16_huffman_infer.huffman_decode.default(
+        A_rem, A_exp, Y, offsets, LUT1, LUT2, LUT3, LUT4, code_lengths)
+
+
+def gemv_bf16_ans(A_rem: Tensor, A_exp: Tensor, X: Tensor, Y: Tensor, offsets: Tensor, LUT: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.gemv_bf16_ans.default(A_rem, A_exp, X, Y, offsets, LUT)
+
+
+def ans_encode(data: Tensor, freq: Tensor, cum: Tensor, output: Tensor, output_lengths: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.ans_encode.default(data, freq, cum, output, output_lengths)
+
+
+def ans_decode(A_rem: Tensor, A_exp: Tensor, Y: Tensor, offsets: Tensor, LUT: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.ans_decode.default(A_rem, A_exp, Y, offsets, LUT)
+
+
+def encode_capacity(n_steps: int) -> int:
+    """Words to reserve per task row of ``huffman_encode``'s output."""
+    return int(_lib.load().bhi_encode_capacity(n_steps))
+
+
+def ans_encode_capacity(n_steps: int) -> int:
+    return int(_lib.load().bhi_ans_encode_capacity(n_steps))

@@ -1,0 +1,117 @@
+/*
+ * bhi.h -- C ABI of libbhi_hip.so: fused entropy-decode + GEMV for compressed BF16
+ * weights on gfx950 (MI355X).
+ *
+ * Each entry point stands in for one torch custom op of the reference
+ * (namespace "bf16_huffman_infer", schemas at
+ * bf16_huffman_infer/src/bf16_huffman_infer.cpp:29-35, CUDA implementations
+ * registered at bf16_huffman_infer/src/kernel.cu:922-930).  The arguments are the
+ * op's tensors as raw device pointers, in the op's order, followed by the
+ * dimensions the reference reads from tensor sizes and the HIP stream the reference
+ * takes from torch (kernel.cu:30-38).
+ *
+ * Rules for every function:
+ *   - all pointers are device pointers valid on the current HIP device;
+ *   - the call only enqueues work on `stream` (a hipStream_t, NULL = default
+ *     stream); it never synchronises, allocates, frees or keeps a pointer;
+ *   - the return value is 0 on success, a negative BHI_E* code for a rejected
+ *     argument, or a positive hipError_t from the launch; bhi_last_error_string()
+ *     describes the last failure on the calling thread.
+ */
+#ifndef BHI_H
+#define BHI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BHI_EINVAL   (-1)   /* bad dimension / null pointer */
+#define BHI_EBATCH   (-2)   /* batch > BHI_MAX_BATCH (reference: STD_TORCH_CHECK, kernel.cu:472,737) */
+#define BHI_ELAYOUT  (-3)   /* table size or chunking does not match the stream format */
+
+#define BHI_MAX_BATCH 8
+
+/* Format and kernel constants, so that host code has one source of truth
+ * (the reference duplicates OP_PER_LANE / ANS_PRECISION in functional.py:15-16 and
+ * kernel.cu:22-25).  Fills out[0..n) with, in order:
+ *   0 format version        1 lanes per wavefront (64)   2 rows per row group (4)
+ *   3 columns per step (128)4 Huffman table index bits   5 init words per lane (3)
+ *   6 header bits per lane  7 max fused batch            8 rANS precision bits
+ *   9 stream alignment in 32-bit words                   10 tail padding words
+ *  11 task target used by bhi_chunks_per_group           12 max steps per task
+ * Returns the number of constants available. */
+int bhi_constants(int32_t* out, int n);
+
+/* Number of independent streams (chunks) a (split, row group) is cut into; a pure
+ * function of the shape shared by encoder, decoder and launch geometry. */
+int bhi_chunks_per_group(int M, int Ks, int split_k);
+
+const char* bhi_last_error_string(void);
+
+/* gemv_bf16_huffman(A_rem, A_exp, X, Y!, offsets, LUT1, LUT2, LUT3, LUT4, code_lengths)
+ * reference: kernel.cu:445-507 (launcher), :419-442 and :46-219 (kernel).
+ *   A_rem   uint8  [split_k, M, Ks]  sign/mantissa plane, lane-ordered
+ *   A_exp   int32  [exp_words]       task streams (exp_words includes the tail pad)
+ *   X       bf16   [batch, split_k*Ks]
+ *   Y       bf16   [batch, M]        written
+ *   offsets int32  [split_k, M]
+ *   LUT1    uint8  [lut1_bytes]      pair decode table, lut1_bytes = 4 << table bits
+ *   LUT2..4, code_lengths uint8 [256] (carried for the op signature; not read) */
+int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64_t exp_words,
+                          const void* X, void* Y, const void* offsets,
+                          const void* LUT1, int64_t lut1_bytes,
+                          const void* LUT2, const void* LUT3, const void* LUT4,
+                          const void* code_lengths,
+                          int split_k, int M, int Ks, int batch, void* stream);
+
+/* huffman_decode(A_rem, A_exp, Y!, offsets, LUT1, LUT2, LUT3, LUT4, code_lengths)
+ * reference: kernel.cu:534-587 (launcher), :510-531 and :222-310 (kernel).
+ *   Y bf16 [M, split_k*Ks] row-major original weight, written. */
+int bhi_huffman_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
+                       void* Y, const void* offsets,
+                       const void* LUT1, int64_t lut1_bytes,
+                       const void* LUT2, const void* LUT3, const void* LUT4,
+                       const void* code_lengths,
+                       int split_k, int M, int Ks, void* stream);
+
+/* huffman_encode(data, LUT, output!, output_lengths!)
+ * reference: kernel.cu:613-644 (launcher), :590-610 (kernel).
+ *   data    uint8  [n_tasks, n_steps, 64, 8]  exponent bytes in lane order
+ *   LUT     uint32 [65537]                    encoder table: code | len<<16, ESC last
+ *   output  int32  [n_tasks, out_stride]      one finished task stream per row, written
+ *   output_lengths int32 [n_tasks]            words used per task (multiple of 4), written
+ * out_stride must be >= bhi_encode_capacity(n_steps). */
+int bhi_huffman_encode(const void* data, const void* LUT, void* output, void* output_lengths,
+                       int n_tasks, int n_steps, int64_t out_stride, void* stream);
+
+/* Worst-case words one task stream of n_steps steps can occupy. */
+int64_t bhi_encode_capacity(int n_steps);
+
+/* gemv_bf16_ans(A_rem, A_exp, X, Y!, offsets, LUT)
+ * reference: kernel.cu:714-764 (launcher), :686-711 and :46-219 (kernel).
+ *   LUT int32 [256]: (sym<<24)|(freq<<12)|rem, rANS precision 8 (functional.py:286-295). */
+int bhi_gemv_bf16_ans(const void* A_rem, const void* A_exp, int64_t exp_words,
+                      const void* X, void* Y, const void* offsets, const void* LUT,
+                      int split_k, int M, int Ks, int batch, void* stream);
+
+/* ans_decode(A_rem, A_exp, Y!, offsets, LUT)
+ * reference: kernel.cu:878-919 (launcher), :851-875 and :222-310 (kernel). */
+int bhi_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
+                   void* Y, const void* offsets, const void* LUT,
+                   int split_k, int M, int Ks, void* stream);
+
+/* ans_encode(data, freq, cum, output!, output_lengths!)
+ * reference: kernel.cu:814-848 (launcher), :767-811 (kernel).
+ *   freq, cum int32 [256] quantised frequencies (sum 256) and their exclusive prefix. */
+int bhi_ans_encode(const void* data, const void* freq, const void* cum,
+                   void* output, void* output_lengths,
+                   int n_tasks, int n_steps, int64_t out_stride, void* stream);
+
+int64_t bhi_ans_encode_capacity(int n_steps);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BHI_H */

@@ -1,0 +1,322 @@
+"""Executable specification of the wave64 compressed-exponent format (oracle; test
+infrastructure only -- the product never imports this file).
+
+The reference stores 64 private bitstreams per row, padded to the longest one
+(``functional.py:129-193``), and decodes them with one 32-lane warp per row
+(``src/kernel.cu:222-310,354-380``).  The HIP kernels of this repository use a
+different private layout with the same planes and the same module buffers:
+
+planes      ``exp`` = BF16 bits 14..7, ``rem`` = sign<<7 | mantissa (reference
+            ``utils.py:7-12``); ``split_k`` contiguous column blocks of ``Ks`` columns
+            (reference ``functional.py:200``).
+row group   4 consecutive rows.  One wavefront decodes one *task* = (split k, row
+            group g, chunk c): rows 4g..4g+3, columns ``k*Ks + 128*t + ...`` for the
+            steps ``t`` of the chunk.
+step        128 columns x 4 rows.  Lane ``l = 4*b + i`` owns row ``4g+i`` and the 8
+            columns ``128*t + 8*b + j`` (j = 0..7): 4 exponent *pairs* per step.
+rem plane   uint8 ``[split_k, M, Ks]``; the ``4*Ks`` bytes of (k, g) hold step ``t``,
+            lane ``l``, column ``j`` at byte ``512*t + 8*l + j``.
+code        one length-limited (<= 12 bit) Huffman code over exponent *pairs*
+            ``a | b<<8`` (a = even column) plus an ESC word; code bits are consumed
+            LSB first.  ``dec`` is the 4096-entry decode table indexed by the next 12
+            stream bits: ``a | b<<16 | len<<24``; ESC entries carry ``0x80`` in the top
+            byte beside the length.  The two raw exponents of an escaped pair are
+            not in the bitstream: they sit in the task's escape list.
+lane bits   bits 0..7 of a lane's bitstring = number of refill loads the lane will
+            make; codes follow from bit 8.  The bitstring is cut into 32-bit words.
+task stream ``[192 init words][refill words][zero pad][escape list]``, a multiple of 4
+            words.  Init: word ``n`` (n < 3) of lane ``l`` at ``64*n + l``.  Refill words
+            are stored in the order the decoder consumes them: after every step,
+            while any lane's cursor has left its current word, each such lane
+            advances one word and -- if it still has refill loads left -- takes the
+            next stream word, lanes in ascending order (a ballot prefix count).  The
+            cursor is ``bit position - 2`` (the decoder keeps its window shifted left
+            by two so that ``window & 0x3FFC`` is the byte address of the table entry),
+            so a lane leaves word ``m`` when ``position - 2 >= 32*(m+1)``.
+            Escape entries ``a | b<<8`` are consumed per step in (pair, lane) order and
+            stored backwards from the end of the task stream.
+offsets     int32 ``[split_k, M]``: word offset of task (k, g, c) at ``[k, 4*g + c]``;
+            tasks are laid out in (k, g, c) order; unused slots are 0.
+
+Pins: ``decode(encode(x)) == x`` on random, heavy-tailed, constant, all-escape and
+boundary inputs, with the encoder (closed-form positions by prefix sums) and the
+decoder (step-by-step simulation of the kernel) sharing no code beyond the
+constants; cross-check against ``ref_layout`` (both must reproduce the same
+original tensor); the HIP encoder must reproduce ``encode`` bit for bit and the
+HIP decoder must reproduce the original tensor.
+"""
+import numpy as np
+
+LANES = 64
+GROUP_ROWS = 4
+LANE_COLS = 8
+STEP_COLS = 128
+PAIRS_PER_STEP = 4
+INIT_WORDS = 3
+HEADER_BITS = 8
+TABLE_BITS = 12
+ESC_FLAG = 0x80
+CURSOR_BIAS = 2            # the decoder's cursor trails the bit position by 2 (pre-shifted window)
+TARGET_TASKS = 4096
+MIN_CHUNK_STEPS = 4
+MAX_CHUNKS = 4
+ALIGN_WORDS = 4
+TAIL_PAD_WORDS = 1024
+ESC_INDEX = 65536          # slot of the ESC code in the encoder table
+
+
+def chunks_per_group(M: int, Ks: int, split_k: int) -> int:
+    """How many independent streams a (split, row group) is cut into."""
+    steps = Ks // STEP_COLS
+    nc = 1
+    while (nc < MAX_CHUNKS and (M // GROUP_ROWS) * split_k * nc < TARGET_TASKS
+           and steps // (nc * 2) >= MIN_CHUNK_STEPS):
+        nc *= 2
+    return nc
+
+
+def chunk_steps(steps: int, nc: int, c: int):
+    return (steps * c) // nc, (steps * (c + 1)) // nc
+
+
+def lane_order(plane: np.ndarray, split_k: int) -> np.ndarray:
+    """[M, K] byte plane -> [split_k, G, S, 64, 8] in (split, group, step, lane, col)."""
+    M, K = plane.shape
+    Ks = K // split_k
+    assert M % GROUP_ROWS == 0 and Ks % STEP_COLS == 0
+    G, S = M // GROUP_ROWS, Ks // STEP_COLS
+    x = plane.reshape(G, GROUP_ROWS, split_k, S, 16, LANE_COLS)      # g i k t b j
+    return np.ascontiguousarray(x.transpose(2, 0, 3, 4, 1, 5)).reshape(split_k, G, S, LANES, LANE_COLS)
+
+
+def lane_order_inverse(x: np.ndarray) -> np.ndarray:
+    split_k, G, S = x.shape[:3]
+    y = x.reshape(split_k, G, S, 16, GROUP_ROWS, LANE_COLS).transpose(1, 4, 0, 2, 3, 5)  # g i k t b j
+    return np.ascontiguousarray(y).reshape(G * GROUP_ROWS, split_k * S * STEP_COLS)
+
+
+def pack_rem(rem: np.ndarray, split_k: int) -> np.ndarray:
+    M, K = rem.shape
+    return lane_order(rem, split_k).reshape(split_k, M, K // split_k)
+
+
+def unpack_rem(rem_packed: np.ndarray) -> np.ndarray:
+    split_k, M, Ks = rem_packed.shape
+    return lane_order_inverse(rem_packed.reshape(split_k, M // GROUP_ROWS, Ks // STEP_COLS, LANES, LANE_COLS))
+
+
+# ----------------------------------------------------------------------------- encoder
+
+def _encode_tasks(sym: np.ndarray, enc: np.ndarray):
+    """sym: uint8 [nt, ns, 64, 8] -> list of nt uint32 streams."""
+    nt, ns = sym.shape[:2]
+    s = sym.astype(np.uint32)
+    pairs = s[..., 0::2] | (s[..., 1::2] << 8)                      # [nt, ns, 64, 4]
+    e = enc[pairs].astype(np.uint64)
+    ln = (e >> np.uint64(16)).astype(np.int64)
+    esc = ln == 0                                                    # [nt, ns, 64, 4]
+    esc_code = np.uint64(int(enc[ESC_INDEX]) & 0xFFFF)
+    esc_len = int(enc[ESC_INDEX]) >> 16
+    assert 1 <= esc_len <= TABLE_BITS
+    code = np.where(esc, esc_code, e & np.uint64(0xFFFF))
+    ln = np.where(esc, esc_len, ln)
+    assert ln.max() <= TABLE_BITS and ln.min() >= 1
+
+    # per-lane bit strings
+    ln_l = ln.transpose(0, 2, 1, 3).reshape(nt, LANES, ns * PAIRS_PER_STEP)
+    code_l = code.transpose(0, 2, 1, 3).reshape(nt, LANES, ns * PAIRS_PER_STEP)
+    end = HEADER_BITS + np.cumsum(ln_l, axis=-1)
+    off = end - ln_l
+    total_bits = end[..., -1]
+    nwords = (total_bits + 31) // 32
+    nref = np.maximum(nwords - INIT_WORDS, 0)
+    assert nref.max() <= 255
+    maxw = max(int(nwords.max()), INIT_WORDS) + 1
+    lw = np.zeros((nt, LANES, maxw), dtype=np.uint64)
+    ti, li, _ = np.indices(off.shape)
+    val = code_l << (off & 31).astype(np.uint64)
+    np.bitwise_or.at(lw, (ti, li, off >> 5), val & np.uint64(0xFFFFFFFF))
+    np.bitwise_or.at(lw, (ti, li, (off >> 5) + 1), val >> np.uint64(32))
+    lw[..., 0] |= nref.astype(np.uint64)
+
+    # refill schedule: cursor word after each step
+    step_bits = ln.sum(axis=-1).transpose(0, 2, 1)                   # [nt, 64, ns]
+    cur = (HEADER_BITS - CURSOR_BIAS + np.cumsum(step_bits, axis=-1)) >> 5   # cursor word after step t
+    prev = np.concatenate([np.zeros((nt, LANES, 1), np.int64), cur[..., :-1]], axis=-1)
+    cross = cur - prev
+    assert cross.max() <= 2
+    loads = np.zeros((nt, ns, 2, LANES), dtype=bool)
+    widx = np.zeros((nt, ns, 2, LANES), dtype=np.int64)
+    for r in range(2):
+        ordinal = prev + r + 1                                       # 1-based crossing number
+        do = (cross > r) & (ordinal <= nref[..., None])
+        loads[:, :, r, :] = do.transpose(0, 2, 1)
+        widx[:, :, r, :] = (ordinal + INIT_WORDS - 1).transpose(0, 2, 1)
+    flat = loads.reshape(nt, -1)
+    pos = np.cumsum(flat, axis=-1) - flat                            # exclusive rank
+    nrefill = flat.sum(axis=-1)
+    assert np.array_equal(nrefill, nref.sum(axis=-1))
+
+    esc_flat = esc.transpose(0, 1, 3, 2).reshape(nt, -1)             # (step, pair, lane) order
+    pair_flat = pairs.transpose(0, 1, 3, 2).reshape(nt, -1)
+    nesc = esc_flat.sum(axis=-1)
+
+    streams = []
+    lane_of = np.broadcast_to(np.arange(LANES), (ns, 2, LANES)).reshape(-1)
+    for t in range(nt):
+        body = INIT_WORDS * LANES + int(nrefill[t]) + int(nesc[t])
+        total = (body + ALIGN_WORDS - 1) // ALIGN_WORDS * ALIGN_WORDS
+        st = np.zeros(total, dtype=np.uint32)
+        for n in range(INIT_WORDS):
+            st[n * LANES:(n + 1) * LANES] = lw[t, :, n].astype(np.uint32)
+        sel = flat[t]
+        st[INIT_WORDS * LANES + pos[t][sel]] = lw[t, lane_of[sel], widx[t].reshape(-1)[sel]].astype(np.uint32)
+        if nesc[t]:
+            st[total - 1 - np.arange(int(nesc[t]))] = pair_flat[t][esc_flat[t]]
+        streams.append(st)
+    return streams
+
+
+def encode(bits: np.ndarray, split_k: int, enc: np.ndarray):
+    """bits: uint16 [M, K] BF16 patterns -> dict(rem, exp, offsets, nc)."""
+    from .planes import split_bf16
+    M, K = bits.shape
+    Ks = K // split_k
+    S = Ks // STEP_COLS
+    G = M // GROUP_ROWS
+    nc = chunks_per_group(M, Ks, split_k)
+    rem, exp = split_bf16(bits)
+    sym = lane_order(exp, split_k)                                   # [k, G, S, 64, 8]
+    per_chunk = []
+    for c in range(nc):
+        t0, t1 = chunk_steps(S, nc, c)
+        per_chunk.append(_encode_tasks(sym[:, :, t0:t1].reshape(split_k * G, t1 - t0, LANES, LANE_COLS), enc))
+    offsets = np.zeros((split_k, M), dtype=np.int64)
+    parts, cursor = [], 0
+    for k in range(split_k):
+        for g in range(G):
+            for c in range(nc):
+                st = per_chunk[c][k * G + g]
+                offsets[k, GROUP_ROWS * g + c] = cursor
+                parts.append(st)
+                cursor += len(st)
+    parts.append(np.zeros(TAIL_PAD_WORDS, dtype=np.uint32))
+    assert cursor + TAIL_PAD_WORDS < 2 ** 31
+    return {
+        "rem": pack_rem(rem, split_k),
+        "exp": np.concatenate(parts).view(np.int32),
+        "offsets": offsets.astype(np.int32),
+        "nc": nc,
+    }
+
+
+# ----------------------------------------------------------------------------- decoder
+
+def _decode_tasks(words: np.ndarray, base: np.ndarray, end: np.ndarray, ns: int, dec: np.ndarray) -> np.ndarray:
+    """Step-by-step model of one wavefront per task.
+
+    words: uint32 flat buffer; base/end: [nt] word offsets of each task stream and of
+    the stream that follows it.  Returns uint8 [nt, ns, 64, 8].
+    """
+    nt = len(base)
+    U = np.uint64
+    lanes = np.arange(LANES)
+    w64 = words.astype(np.uint64)
+    lo = w64[base[:, None] + lanes]
+    hi = w64[base[:, None] + LANES + lanes]
+    nx = w64[base[:, None] + 2 * LANES + lanes]
+    left = (lo & U(0xFF)).astype(np.int64)
+    c = np.full((nt, LANES), HEADER_BITS - CURSOR_BIAS, dtype=np.int64)
+    ptr = np.zeros(nt, dtype=np.int64)
+    eptr = np.zeros(nt, dtype=np.int64)
+    out = np.zeros((nt, ns, LANES, LANE_COLS), dtype=np.uint8)
+    dec64 = dec.astype(np.uint64)
+    M32 = U(0xFFFFFFFF)
+    for t in range(ns):
+        cu = c.astype(np.uint64)
+        wlo = (((hi << U(32)) | lo) >> cu) & M32
+        whi = (((nx << U(32)) | hi) >> cu) & M32
+        win = (whi << U(32)) | wlo
+        used = np.zeros((nt, LANES), dtype=np.int64)
+        for q in range(PAIRS_PER_STEP):
+            e = dec64[((win >> U(CURSOR_BIAS)) & U((1 << TABLE_BITS) - 1)).astype(np.int64)]
+            ln = ((e >> U(24)) & U(0x7F)).astype(np.int64)
+            esc = ((e >> U(31)) & U(1)).astype(bool)
+            a = (e & U(0xFF)).astype(np.uint8)
+            b = ((e >> U(16)) & U(0xFF)).astype(np.uint8)
+            if esc.any():
+                rank = np.cumsum(esc, axis=-1) - esc
+                src = end[:, None] - 1 - (eptr[:, None] + rank)
+                v = words[np.where(esc, src, 0)]
+                a = np.where(esc, (v & 0xFF).astype(np.uint8), a)
+                b = np.where(esc, ((v >> 8) & 0xFF).astype(np.uint8), b)
+                eptr += esc.sum(axis=-1)
+            out[:, t, :, 2 * q] = a
+            out[:, t, :, 2 * q + 1] = b
+            win = win >> ln.astype(np.uint64)
+            used += ln
+        c += used
+        assert c.max() < 96
+        while (c >= 32).any():
+            cross = c >= 32
+            c = np.where(cross, c - 32, c)
+            lo = np.where(cross, hi, lo)
+            hi = np.where(cross, nx, hi)
+            load = cross & (left > 0)
+            rank = np.cumsum(load, axis=-1) - load
+            src = base[:, None] + INIT_WORDS * LANES + ptr[:, None] + rank
+            nx = np.where(load, w64[np.where(load, src, 0)], nx)
+            left -= load
+            ptr += load.sum(axis=-1)
+    assert (left == 0).all()
+    return out
+
+
+def decode(rem_packed: np.ndarray, exp_words: np.ndarray, offsets: np.ndarray, dec: np.ndarray) -> np.ndarray:
+    """-> uint16 [M, K] BF16 patterns."""
+    from .planes import rebuild_bf16
+    split_k, M, Ks = rem_packed.shape
+    S, G = Ks // STEP_COLS, M // GROUP_ROWS
+    nc = chunks_per_group(M, Ks, split_k)
+    words = exp_words.view(np.uint32)
+    total = len(words) - TAIL_PAD_WORDS
+    off = offsets.astype(np.int64).reshape(split_k, G, GROUP_ROWS)[:, :, :nc]   # [k, G, nc] in layout order
+    flat = off.reshape(-1)
+    nxt = np.concatenate([flat[1:], [total]]).reshape(off.shape)
+    sym = np.zeros((split_k, G, S, LANES, LANE_COLS), dtype=np.uint8)
+    for c in range(nc):
+        t0, t1 = chunk_steps(S, nc, c)
+        r = _decode_tasks(words, off[:, :, c].reshape(-1), nxt[:, :, c].reshape(-1), t1 - t0, dec)
+        sym[:, :, t0:t1] = r.reshape(split_k, G, t1 - t0, LANES, LANE_COLS)
+    exp = lane_order_inverse(sym)
+    rem = unpack_rem(rem_packed)
+    return rebuild_bf16(rem, exp)
+
+
+# ----------------------------------------------------------------------------- table checks
+
+def check_tables(dec: np.ndarray, enc: np.ndarray) -> None:
+    """Consistency of a decode table with its encoder table (raises AssertionError).
+
+    Every 12-bit index must resolve to exactly the pair (or ESC) whose LSB-first code
+    is a prefix of the index; the code is therefore prefix-free and complete.
+    """
+    assert dec.shape == (1 << TABLE_BITS,) and enc.shape == (ESC_INDEX + 1,)
+    covered = np.zeros(1 << TABLE_BITS, dtype=np.int64)
+    present = np.nonzero(enc >> 16)[0]
+    kraft = 0.0
+    for p in present:
+        code, ln = int(enc[p]) & 0xFFFF, int(enc[p]) >> 16
+        assert 1 <= ln <= TABLE_BITS and code < (1 << ln)
+        kraft += 2.0 ** -ln
+        idx = code + (np.arange(1 << (TABLE_BITS - ln)) << ln)
+        covered[idx] += 1
+        got = dec[idx]
+        if p == ESC_INDEX:
+            assert (got >> 24 == (ln | ESC_FLAG)).all()
+        else:
+            want = (p & 0xFF) | ((p >> 8) << 16) | (ln << 24)
+            assert (got == want).all(), (p, ln)
+    assert (covered == 1).all()
+    assert abs(kraft - 1.0) < 1e-9
+    assert enc[ESC_INDEX] >> 16 != 0

@@ -1,0 +1,98 @@
+"""HIP Huffman path against the oracle and against the original tensors (needs a GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (bits_of, gaussian_weight, pair_counts, random_bits_weight, special_values_weight,
+                     student_t_weight)
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-3        # GEMV tolerance against fp32 accumulation of the same BF16 operands
+
+MAKERS = {
+    "gauss": gaussian_weight,
+    "t3": student_t_weight,
+    "bits": random_bits_weight,
+    "special": special_values_weight,
+    "zeros": lambda M, K, seed=0: torch.zeros(M, K, dtype=torch.bfloat16),
+}
+
+
+def _compress(w, n=None):
+    from bf16_huffman_infer_amd.functional import HuffmanWeight
+    return HuffmanWeight.compress(w) if n is None else HuffmanWeight.compress_split_n(w, n=n)
+
+
+@pytest.mark.parametrize("kind,M,K,n", [
+    ("gauss", 128, 384, None), ("gauss", 256, 512, 2), ("t3", 128, 1024, None), ("bits", 128, 256, None),
+    ("special", 256, 1280, None), ("zeros", 128, 128 * 3, None), ("gauss", 1024, 4096, None),
+    ("gauss", 128, 2048, 4),
+])
+def test_encoder_matches_oracle_and_decodes(cuda, kind, M, K, n):
+    """HIP encoder == numpy encoder bit for bit; HIP decoder == original tensor."""
+    from bf16_huffman_infer_amd.huffman import LUTHuffmanEncoder
+    from bf16_huffman_infer_amd.utils import get_block_size_n
+    from oracle import wave64
+    w = MAKERS[kind](M, K, seed=3)
+    mod = _compress(w, n)
+    split_k = n or get_block_size_n(w)[0]
+    assert tuple(mod.rem.shape) == (split_k, M, K // split_k) and mod.rem.dtype == torch.uint8
+    assert tuple(mod.offsets.shape) == (split_k, M) and mod.offsets.dtype == torch.int32
+    assert mod.exp.dtype == torch.int32 and mod.LUT1.numel() == 16384
+
+    codec = LUTHuffmanEncoder()
+    codec.build_lut(pair_counts(bits_of(w)))
+    assert np.array_equal(codec.LUT1, mod.LUT1.numpy())
+    want = wave64.encode(bits_of(w), split_k, codec.enc_table)
+    assert np.array_equal(want["rem"], mod.rem.numpy())
+    assert np.array_equal(want["offsets"], mod.offsets.numpy())
+    assert np.array_equal(want["exp"], mod.exp.numpy())
+
+    mod = mod.cuda()
+    got = mod.get_weight()
+    assert got.shape == w.shape and got.dtype == torch.bfloat16
+    assert torch.equal(got.view(torch.int16).cpu(), w.view(torch.int16))
+
+
+@pytest.mark.parametrize("bs", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("kind,M,K,n", [("gauss", 256, 1024, None), ("t3", 128, 512, 2), ("bits", 128, 256, None)])
+def test_fused_gemv_matches_fp32(cuda, kind, M, K, n, bs):
+    w = MAKERS[kind](M, K, seed=5)
+    if kind == "bits":                      # keep the reference product finite
+        w = (w.float().nan_to_num(0.0, 0.0, 0.0).clamp(-1, 1)).bfloat16()
+    mod = _compress(w, n).cuda()
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(bs, K, generator=g).bfloat16().cuda()
+    y = torch.nn.functional.linear(x, mod)
+    assert y.shape == (bs, M) and y.dtype == torch.bfloat16
+    ref = x.float() @ w.cuda().float().T
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+
+
+def test_large_batch_falls_back_to_decode_then_gemm(cuda):
+    from bf16_huffman_infer_amd.functional import CompressedLinear
+    w = gaussian_weight(256, 512, seed=7)
+    bias = torch.randn(256).bfloat16()
+    lin = CompressedLinear(_compress(w), bias).cuda()
+    x = torch.randn(3, 5, 512).bfloat16().cuda()            # 15 rows > 8
+    y = lin(x)
+    ref = torch.nn.functional.linear(x, w.cuda(), bias.cuda())
+    assert y.shape == (3, 5, 256)
+    torch.testing.assert_close(y.float(), ref.float(), rtol=RTOL, atol=ATOL)
+    y8 = lin(x[:1])                                          # 5 rows: fused path + bias
+    torch.testing.assert_close(y8.float(), ref[:1].float(), rtol=RTOL, atol=5e-3)
+
+
+def test_ops_reject_cpu_tensors_and_big_batch(cuda):
+    from bf16_huffman_infer_amd import ops
+    mod = _compress(gaussian_weight(128, 256, seed=1))
+    y = torch.empty(128, 256, dtype=torch.bfloat16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        ops.huffman_decode(mod.rem, mod.exp, y, mod.offsets, mod.LUT1, mod.LUT2, mod.LUT3, mod.LUT4, mod.code_lengths)
+    mod = mod.cuda()
+    x = torch.zeros(9, 1, 256, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty(9, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="batch"):
+        ops.gemv_bf16_huffman(mod.rem, mod.exp, x, out, mod.offsets, mod.LUT1, mod.LUT2, mod.LUT3, mod.LUT4,
+                              mod.code_lengths)
