@@ -1,0 +1,206 @@
+"""Fused decode-GEMV benchmark on one MI355X.
+
+Workload: the linear layers of one Qwen2.5-7B decoder block (q/k/v fused 3584->4608,
+o 3584->3584, gate and up 3584->18944, down 18944->3584), BF16 weights iid N(0, 0.02)
+from a seed, Huffman-compressed, batch 1.  One step = one fused decode-GEMV launch per
+layer.  Two independently seeded copies of the block alternate between steps so that
+the 256 MB last-level cache cannot serve the weights.
+
+Prints one JSON line: whole-block GB/s on compressed bytes, with the roofline of the
+dominant kernel (the 18944x3584 GEMV) and the CPU baseline (the reference's layout and
+decoder restated in numpy + a host matmul, timed on this machine).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+LAYERS = [("qkv_proj", 4608, 3584), ("o_proj", 3584, 3584), ("gate_proj", 18944, 3584),
+          ("up_proj", 18944, 3584), ("down_proj", 3584, 18944)]
+COPIES = 2
+STD = 0.02
+
+
+def make_weight(M, K, seed, device):
+    g = torch.Generator(device=device).manual_seed(seed)
+    return (torch.randn(M, K, generator=g, device=device) * STD).bfloat16()
+
+
+def weight_bytes(mod) -> int:
+    return sum(b.nelement() * b.element_size() for b in mod.buffers())
+
+
+def gemv_bytes(mod, bs, M, K) -> int:
+    """Algorithmic bytes of one fused GEMV: every weight-module buffer once + X + Y."""
+    return weight_bytes(mod) + bs * K * 2 + bs * M * 2
+
+
+def build_block(algo, device, copy):
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight
+    cls = {"huffman": HuffmanWeight, "ans": ANSWeight}[algo]
+    mods = []
+    for i, (name, M, K) in enumerate(LAYERS):
+        w = make_weight(M, K, 1000 * copy + i, device)
+        mods.append(cls.compress(w).to(device))
+        del w
+    return mods
+
+
+def time_launches(fn, n, warmup, launches_per_graph=1):
+    """Seconds per call of ``fn``.  ``fn`` is captured once into a HIP graph (as the decode
+    step is in serving, and as the reference's own benchmark does with CUDA graphs) so
+    that the Python dispatch cost of the op wrappers is not what gets timed; the graph
+    holds ``launches_per_graph`` consecutive calls."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            for _ in range(launches_per_graph):
+                fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(launches_per_graph):
+            fn()
+    replays = max(1, (n + launches_per_graph - 1) // launches_per_graph)
+    for _ in range(max(1, warmup // launches_per_graph)):
+        graph.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / (replays * launches_per_graph)
+
+
+def cpu_baseline(rows=4096, K=3584, reps=3):
+    """Reference layout + reference decoder (numpy) + host matmul on a slice of gate_proj."""
+    import numpy as np
+    from oracle import planes, ref_layout, ref_tables
+    g = torch.Generator().manual_seed(2)
+    w = (torch.randn(rows, K, generator=g) * STD).bfloat16()
+    bits = w.view(torch.int16).numpy().view(np.uint16)
+    _, exp = planes.split_bf16(bits)
+    luts, lens, codes = ref_tables.build_cascade_luts(np.bincount(exp.reshape(-1), minlength=256))
+    enc = ref_layout.encode(bits, 1, "huffman", codes)
+    x = torch.randn(1, K, generator=g).bfloat16()
+    nbytes = enc["rem"].nbytes + enc["exp"].nbytes + enc["offsets"].nbytes + 5 * 256 + K * 2 + rows * 2
+    times = []
+    for _ in range(reps):
+        t = time.perf_counter()
+        dec = ref_layout.decode_huffman(enc["rem"], enc["exp"], enc["offsets"], luts, lens)
+        t_dec = time.perf_counter() - t
+        wd = torch.from_numpy(dec.view(np.int16)).view(torch.bfloat16)
+        t = time.perf_counter()
+        y = (x.float() @ wd.float().T).bfloat16()
+        t_mm = time.perf_counter() - t
+        times.append((t_dec + t_mm, t_dec, t_mm))
+    assert np.array_equal(dec, bits), "CPU baseline decoder is not lossless"
+    times.sort()
+    total, t_dec, t_mm = times[len(times) // 2]
+    return {
+        "value": round(nbytes / total / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"first {rows} rows of gate_proj ({rows}x{K}), reference layout; numpy decode {t_dec:.2f}s "
+                  f"(1 thread) + torch matmul {t_mm * 1e3:.1f}ms ({torch.get_num_threads()} threads); "
+                  f"os.cpu_count()={os.cpu_count()}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--algo", default="huffman", choices=["huffman", "ans"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+
+    from bf16_huffman_infer_amd import _lib
+    _lib.load()                                   # fail before any work if the HIP library is missing
+    import torch.nn.functional as F
+
+    device = torch.device("cuda", 0)
+    bs = args.batch
+    blocks = [build_block(args.algo, device, c) for c in range(COPIES)]
+    xs = [torch.randn(bs, K, device=device).bfloat16() for _, _, K in LAYERS]
+    block_bytes = sum(gemv_bytes(m, bs, M, K) for m, (_, M, K) in zip(blocks[0], LAYERS))
+    raw_bytes = sum(M * K * 2 for _, M, K in LAYERS)
+
+    # parity gate inside the benchmark: one layer must decode bit-exactly
+    w0 = make_weight(LAYERS[1][1], LAYERS[1][2], 1, device)
+    assert torch.equal(blocks[0][1].get_weight().view(torch.int16), w0.view(torch.int16)), "decode is not lossless"
+    del w0
+
+    state = {"i": 0}
+
+    def step():
+        mods = blocks[state["i"] % COPIES]
+        state["i"] += 1
+        for m, x in zip(mods, xs):
+            F.linear(x, m)
+
+    sec = time_launches(step, args.steps, args.warmup, launches_per_graph=COPIES)
+    gbs = block_bytes / sec / 1e9
+
+    # per-layer timing and the roofline of the dominant kernel
+    per_layer = {}
+    for li, (name, M, K) in enumerate(LAYERS):
+        st = {"i": 0}
+
+        def one(li=li, st=st):
+            F.linear(xs[li], blocks[st["i"] % COPIES][li])
+            st["i"] += 1
+        per_layer[name] = time_launches(one, max(50, args.steps), args.warmup, launches_per_graph=COPIES)
+    big = [2, 3]                                  # gate and up of both copies: four distinct 96 MB streams
+    st = {"i": 0}
+
+    def dominant():
+        i = st["i"]
+        F.linear(xs[big[i % 2]], blocks[(i // 2) % COPIES][big[i % 2]])
+        st["i"] += 1
+    t_dom = time_launches(dominant, max(100, args.steps), args.warmup, launches_per_graph=2 * COPIES)
+    dom_bytes = gemv_bytes(blocks[0][2], bs, LAYERS[2][1], LAYERS[2][2])
+    achieved = dom_bytes / t_dom / 1e9
+
+    out = {
+        "metric": "fused decode-GEMV GB/s (compressed bytes, % HBM peak); bs=1 tokens/s",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"Qwen2.5-7B decoder-block linears (qkv 4608x3584, o 3584x3584, gate/up 18944x3584, "
+                               f"down 3584x18944), N(0,0.02) seeded, algo={args.algo}, batch={bs}, {COPIES} "
+                               f"alternating weight copies"},
+        "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "compressed_bytes_per_step": block_bytes, "compression_ratio": round(
+            sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),
+        "block_steps_per_s": round(1.0 / sec, 1),
+        "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
+        "roofline": {"bound": "hbm", "kernel": f"gemv_huffman_kernel<{bs}> 18944x3584" if args.algo == "huffman"
+                     else f"gemv_ans_kernel<{bs}> 18944x3584",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": dom_bytes, "us_per_launch": round(t_dom * 1e6, 2)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -55,7 +55,7 @@ def check(rc: int, what: str) -> None:
 
 
 _CONST_NAMES = (
-    "format_version", "lanes", "group_rows", "step_cols", "table_bits", "init_words",
+    "format_version", "lanes", "group_rows", "step_cols", "table_bits", "window_words",
     "header_bits", "max_batch", "ans_precision", "align_words", "tail_pad_words",
     "target_tasks", "max_task_steps",
 )

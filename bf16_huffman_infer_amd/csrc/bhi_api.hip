@@ -22,7 +22,7 @@ extern "C" const char* bhi_last_error_string(void) { return g_err; }
 extern "C" int bhi_constants(int32_t* out, int n) {
     const int32_t v[] = {
         bhi::kFormatVersion, bhi::kLanes, bhi::kGroupRows, bhi::kStepCols, bhi::kTableBits,
-        bhi::kInitWords, bhi::kHeaderBits, bhi::kMaxBatch, bhi::kAnsPrecision,
+        bhi::kWindowWords, bhi::kHeaderBits, bhi::kMaxBatch, bhi::kAnsPrecision,
         bhi::kAlignWords, bhi::kTailPadWords, bhi::kTargetTasks, bhi::kMaxTaskSteps,
     };
     const int total = (int)(sizeof(v) / sizeof(v[0]));

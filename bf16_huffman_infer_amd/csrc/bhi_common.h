@@ -3,14 +3,11 @@
 // Stream format in one paragraph (the numpy model under oracle/ is the executable
 // statement): a task = (split k, 4-row group g, chunk c).  One wavefront decodes one
 // task.  Per step every lane l = 4*b + i owns row 4g+i and the 8 columns
-// 128*t + 8*b + j, i.e. four exponent pairs.  A lane's code bits start at bit 8 of its
-// private bitstring (bits 0..7 = number of refill loads it will make); the bitstring is
-// cut into 32-bit words; words 0..2 of lane l sit at [l], [64+l], [128+l] of the task
-// stream and all later words are stored in the order the wavefront consumes them:
-// after each step, while any lane's cursor has left its word, those lanes advance one
-// word and the ones that still have loads left take consecutive stream words in lane
-// order.  Escaped pairs keep only the ESC code in band; their two bytes are read
-// backwards from the end of the task stream in (pair, lane) order.
+// 128*t + 8*b + j, i.e. four exponent pairs.  A lane's code bits start at bit 2 of its
+// private bitstring, the bitstring is cut into 32-bit words, and word w of lane l sits
+// at [64*w + l] of the task block ("row" w); the block has as many rows as its longest
+// lane.  Escaped pairs keep only the ESC code in band; their two bytes are read
+// backwards from the end of the task block in (pair, lane) order.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -23,16 +20,15 @@ constexpr int kGroupRows = 4;
 constexpr int kLaneCols = 8;
 constexpr int kStepCols = 128;
 constexpr int kPairsPerStep = 4;
-constexpr int kInitWords = 3;
-constexpr int kHeaderBits = 8;
-constexpr int kCursorBias = 2;
+constexpr int kWindowWords = 3;
+constexpr int kHeaderBits = 2;
 constexpr int kTableBits = 12;
 constexpr int kTableEntries = 1 << kTableBits;
 constexpr uint32_t kTableMask = (kTableEntries - 1) << 2;   // byte address mask
 constexpr int kMaxBatch = 8;
 constexpr int kAnsPrecision = 8;
 constexpr int kAlignWords = 4;
-constexpr int kTailPadWords = 1024;
+constexpr int kTailPadWords = 2048;
 constexpr int kTargetTasks = 4096;
 constexpr int kMinChunkSteps = 4;
 constexpr int kMaxChunks = 4;
@@ -57,11 +53,15 @@ __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_bal
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
-// Two BF16 values from (table entry, rem bytes).  `e` holds exponent a in bits 7..0 and
-// exponent b in bits 23..16; `z` holds [rb, rb, ra, ra]: the sign comes from the upper
-// copy of each rem byte, the mantissa from the lower copy, the exponent from e<<7.
+// Table entry: len in bits 4..0, ESC flag in bit 15, exponent a in bits 14..7 and
+// exponent b in bits 30..23 -- where a packed pair of BF16 values keeps them.
+constexpr uint32_t kLenMask = 0x801Fu;       // length and ESC flag
+constexpr uint32_t kEscStep = 0x8000u;       // what an ESC entry adds to the cursor
+
+// Two BF16 values from (table entry, rem bytes).  `z` holds [rb, rb, ra, ra]: the sign
+// comes from the upper copy of each rem byte, the mantissa from the lower copy.
 __device__ __forceinline__ uint32_t rebuild_pair(uint32_t e, uint32_t z) {
-    return ((e << 7) & 0x7F807F80u) | (z & 0x807F807Fu);
+    return (e & 0x7F807F80u) | (z & 0x807F807Fu);
 }
 
 __device__ __forceinline__ uint32_t rem_lo_pair(uint32_t r) { return __builtin_amdgcn_perm(r, r, 0x01010000u); }
@@ -82,76 +82,149 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
     return s;
 }
 
-// Per-lane Huffman bit cursor over the wavefront's shared stream.
-struct HuffCursor {
-    uint32_t lo, hi, nx;     // three consecutive words of this lane's bitstring
-    uint32_t c;              // cursor = bit position - 2 inside `lo`, < 32 between steps
-    uint32_t left;           // refill loads this lane still has to make
-    uint32_t ptr;            // wave-uniform: next unread refill word of the task stream
-    uint32_t eptr;           // wave-uniform: escape entries consumed so far
-    const uint32_t* sp;      // task stream
-    const uint32_t* ep;      // one past the task stream (escape list grows down from here)
+// A task is processed in segments of kSegSteps steps: load phase (every global load of
+// the segment issued back to back, unconditionally, with clamped indices), then compute
+// phase (no global loads).  VMEM loads complete in issue order, so a load placed inside
+// the compute phase would make its wait drain the whole queue; latency is hidden by the
+// other wavefronts of the SIMD being in a different phase.
+//
+// Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each).
+// Row r lives in slot r % kRingRows; slots 0 and 1 are mirrored behind the last slot so
+// that the three rows of a lane's window are always at +0, +256 and +512 bytes.  Lanes
+// sit at different rows, yet row r of lane l is always in bank l % 32: window reads are
+// conflict free.  The ring is topped up when some lane's window is about to leave the
+// staged rows (a cheap per-step test); a lane that is more than a ring ahead of the
+// slowest lane reads its window from global memory instead.
+constexpr int kSegSteps = 8;
+constexpr int kRingRows = 16;
+constexpr int kRingSlots = kRingRows + 2;
+constexpr int kRingWords = kRingSlots * kLanes;
 
-    __device__ __forceinline__ void init(const uint32_t* __restrict__ words, TaskSpan span, int lane) {
-        sp = words + span.base;
+// LDS pointers are kept in their own address space: a pointer that may be LDS or global
+// turns every access into a flat load, which waits on the global-memory counter.
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+
+__device__ __forceinline__ uint32_t wave_min(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        uint32_t u = (uint32_t)__shfl_xor((int)v, o);
+        v = u < v ? u : v;
+    }
+    return v;
+}
+
+// Per-lane Huffman bit cursor over the lane's rows of the task block.
+struct HuffCursor {
+    uint32_t pos;            // bit position - 2 (the window is kept shifted left by two)
+    uint32_t rhi;            // wave-uniform: rows [0, rhi) have been staged
+    uint32_t lim;            // wave-uniform: windows starting below this bit are fully staged
+    uint32_t nrows;          // wave-uniform: rows of the block worth staging
+    uint32_t eptr;           // wave-uniform: escape entries consumed so far
+    const uint32_t* bp;      // task block, this lane's column
+    const uint32_t* ep;      // one past the task block (escape list grows down from here)
+    lds_u32* ring;           // this wavefront's LDS ring, this lane's column
+
+    __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t* ring_) {
+        bp = words + span.base + lane;
         ep = words + span.end;
-        lo = sp[lane];
-        hi = sp[kLanes + lane];
-        nx = sp[2 * kLanes + lane];
-        left = lo & 0xFFu;
-        c = kHeaderBits - kCursorBias;
-        ptr = kInitWords * kLanes;
+        ring = (lds_u32*)ring_ + lane;
+        nrows = uniform((span.end - span.base + kLanes - 1) / kLanes);
+        pos = 0;
+        rhi = 0;
+        lim = 0;
         eptr = 0;
     }
 
-    // Decode the four pairs of one step.  e[q] = a | b<<16 | (len|esc<<7)<<24.
-    // `nx` is first needed after the second lookup, two LDS round trips after the
-    // refill of the previous step issued its load.
+    // Stage rows up to kRingRows past the slowest lane.  Global loads + LDS stores.
+    __device__ __forceinline__ void top_up() {
+        const uint32_t mmin = uniform(wave_min(pos) >> 5);
+        uint32_t hi = mmin + kRingRows;
+        hi = hi < nrows ? hi : nrows;
+        uint32_t v[kRingRows];
+#pragma unroll
+        for (int j = 0; j < kRingRows; ++j)
+            if (rhi + j < hi) v[j] = bp[(size_t)(rhi + j) * kLanes];
+#pragma unroll
+        for (int j = 0; j < kRingRows; ++j) {
+            if (rhi + j < hi) {
+                const uint32_t slot = (rhi + j) & (kRingRows - 1);
+                ring[slot * kLanes] = v[j];
+                if (slot < 2) ring[(kRingRows + slot) * kLanes] = v[j];
+            }
+        }
+        rhi = hi > rhi ? hi : rhi;
+        // windows read rows m..m+2; once the whole block is staged nothing can be missing
+        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi >= 2 ? (rhi - 2) << 5 : 0u);
+    }
+
+    // Decode the four pairs of one step; e[q] are raw table entries.
+    template <bool HAS_ESC>
     __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
+        uint32_t lo, hi, nx;
+        if (__builtin_expect(ballot(pos >= lim) != 0, 0)) {
+            top_up();
+            fetch_slow(lo, hi, nx);
+        } else {
+            const lds_u32* w = ring + ((pos >> 5) & (kRingRows - 1)) * kLanes;
+            lo = w[0];
+            hi = w[kLanes];
+            nx = w[2 * kLanes];
+        }
         const char* tb = (const char*)table;
-        uint32_t wlo = __builtin_amdgcn_alignbit(hi, lo, c);
+        const uint32_t c = pos & 31u;
+        const uint32_t wlo = __builtin_amdgcn_alignbit(hi, lo, c);
         e[0] = *(const uint32_t*)(tb + (wlo & kTableMask));
-        uint32_t l0 = e[0] >> 24;
-        uint32_t w1 = wlo >> (l0 & 31u);
+        const uint32_t w1 = wlo >> (e[0] & 31u);
         e[1] = *(const uint32_t*)(tb + (w1 & kTableMask));
-        uint32_t s01 = l0 + (e[1] >> 24);
-        uint32_t whi = __builtin_amdgcn_alignbit(nx, hi, c);
-        uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, s01);
-        e[2] = *(const uint32_t*)(tb + (w2 & kTableMask));
-        uint32_t l2 = e[2] >> 24;
-        uint32_t w3 = w2 >> (l2 & 31u);
-        e[3] = *(const uint32_t*)(tb + (w3 & kTableMask));
-        c += s01 + l2 + (e[3] >> 24);
-        if (__builtin_expect(ballot(c >= 128u) != 0, 0)) escapes(e);
-        // a step consumes at most 48 bits, so a lane leaves at most two words
-        if (ballot(c >= 32u) != 0) {
-            refill_round();
-            if (__builtin_expect(ballot(c >= 32u) != 0, 0)) refill_round();
+        const uint32_t whi = __builtin_amdgcn_alignbit(nx, hi, c);
+        if (HAS_ESC) {
+            const uint32_t s01 = (e[0] & kLenMask) + (e[1] & kLenMask);
+            const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, s01);
+            e[2] = *(const uint32_t*)(tb + (w2 & kTableMask));
+            const uint32_t w3 = w2 >> (e[2] & 31u);
+            e[3] = *(const uint32_t*)(tb + (w3 & kTableMask));
+            const uint32_t sum = s01 + (e[2] & kLenMask) + (e[3] & kLenMask);
+            pos += sum & 0x3Fu;
+            if (__builtin_expect(ballot(sum >= kEscStep) != 0, 0)) escapes(e);
+        } else {
+            // lengths sit in bits 4..0 and bits 5, 6 are clear, so the low six bits of a
+            // sum of raw entries are the sum of the lengths (at most 48)
+            const uint32_t t01 = e[0] + e[1];
+            const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, t01);
+            e[2] = *(const uint32_t*)(tb + (w2 & kTableMask));
+            const uint32_t w3 = w2 >> (e[2] & 31u);
+            e[3] = *(const uint32_t*)(tb + (w3 & kTableMask));
+            pos += (t01 + e[2] + e[3]) & 0x3Fu;
         }
     }
 
-    // ESC entries carry 0x80 in the length byte, so every escaped pair added 128 to c.
+    // After a top-up: lanes whose window is staged read the ring, the others (more than
+    // a ring ahead of the slowest lane) read global memory.
+    __device__ __forceinline__ void fetch_slow(uint32_t& lo, uint32_t& hi, uint32_t& nx) {
+        const uint32_t m = pos >> 5;
+        const bool staged = pos < lim;
+        // clamp so that both reads are always in range, then pick per lane
+        const lds_u32* w = ring + (m & (kRingRows - 1)) * kLanes;
+        const uint32_t l0 = w[0], l1 = w[kLanes], l2 = w[2 * kLanes];
+        const uint32_t* g = bp + (size_t)(staged ? 0u : m) * kLanes;
+        const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
+        lo = staged ? l0 : g0;
+        hi = staged ? l1 : g1;
+        nx = staged ? l2 : g2;
+    }
+
+    // Exponents of escaped pairs come from the escape list, in (pair, lane) order.
     __device__ __forceinline__ void escapes(uint32_t (&e)[4]) {
-        c &= 127u;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            bool esc = (e[q] >> 31) != 0;
+            bool esc = (e[q] & kEscStep) != 0;
             uint64_t m = ballot(esc);
             if (esc) {
                 uint32_t v = *(ep - 1 - (eptr + lane_rank(m)));
-                e[q] = (v & 0xFFu) | ((v & 0xFF00u) << 8);
+                e[q] = ((v & 0xFFu) << 7) | ((v & 0xFF00u) << 15);
             }
             eptr = uniform(eptr + (uint32_t)__builtin_popcountll(m));
         }
-    }
-
-    __device__ __forceinline__ void refill_round() {
-        const bool cross = c >= 32u;
-        if (cross) { c -= 32u; lo = hi; hi = nx; }
-        const bool load = cross && left != 0;
-        const uint64_t m = ballot(load);
-        if (load) { nx = sp[ptr + lane_rank(m)]; left -= 1; }
-        ptr = uniform(ptr + (uint32_t)__builtin_popcountll(m));
     }
 };
 

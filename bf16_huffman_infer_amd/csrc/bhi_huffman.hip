@@ -10,11 +10,8 @@
 
 namespace bhi {
 
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, x), acc, false);
-}
+typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // Cooperative copy of the 16 KB pair table into LDS.
 __device__ __forceinline__ void load_table(uint32_t* __restrict__ lds, const uint32_t* __restrict__ g) {
@@ -28,12 +25,160 @@ struct Shape {
     uint32_t total_words;
 };
 
+// Runs one task segment by segment.  A policy supplies the operands that travel with
+// the exponent stream: `Slot` holds what is loaded for a whole segment in the load
+// phase (`load(slot, t)`, t clamped by the policy); `take(...)` hands out what the
+// policy pipelines on its own inside the compute phase; `use(...)` receives the
+// lane's four rebuilt BF16 pairs (columns 0..7 of its row in step t).
+template <bool HAS_ESC, class Policy>
+__device__ __forceinline__ void run_task(HuffCursor& cur, const uint32_t* lut, Policy& pol, int ns) {
+    pol.prime();
+    for (int seg = 0; seg < ns; seg += kSegSteps) {
+        // ---- load phase: nothing but global loads, all unconditional
+        typename Policy::Slot slot[kSegSteps];
+#pragma unroll
+        for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], seg + i);
+        // ---- compute phase
+#pragma unroll
+        for (int i = 0; i < kSegSteps; ++i) {
+            if (seg + i < ns) {
+                const typename Policy::Piped piped = pol.take(slot[i], i, seg + i);
+                uint32_t e[4];
+                cur.template step<HAS_ESC>(lut, e);
+                uint32_t w[4];
+                const uint2 r = slot[i].rem;
+                w[0] = rebuild_pair(e[0], rem_lo_pair(r.x));
+                w[1] = rebuild_pair(e[1], rem_hi_pair(r.x));
+                w[2] = rebuild_pair(e[2], rem_lo_pair(r.y));
+                w[3] = rebuild_pair(e[3], rem_hi_pair(r.y));
+                pol.use(piped, seg + i, w);
+            }
+        }
+    }
+}
+
+// The format header (code_lengths buffer): [0] version, [1] table bits, [2] ESC code
+// length, [3] nonzero when the matrix contains escaped pairs.
+__device__ __forceinline__ bool header_has_esc(const uint8_t* __restrict__ header) {
+    return uniform(header[3]) != 0;
+}
+
+// decode-to-BF16: rem in, 16 bytes of weights out per lane and step
+struct StorePolicy {
+    struct Slot { uint2 rem; };
+    struct Piped {};
+    const uint2* rem0;       // this lane's 8 rem bytes of the task's first step
+    uint16_t* yp;            // this lane's 8 output columns of the task's first step
+    int last;
+
+    __device__ __forceinline__ void prime() const {}
+    __device__ __forceinline__ void load(Slot& s, int t) const {
+        t = t < last ? t : last;
+        s.rem = rem0[(size_t)t * kLanes];
+    }
+    __device__ __forceinline__ Piped take(const Slot&, int, int) const { return Piped{}; }
+    __device__ __forceinline__ void use(const Piped&, int t, const uint32_t (&w)[4]) const {
+        *(uint4*)(yp + (size_t)t * kStepCols) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+};
+
+// Broadcast of lane q of every quad (dpp quad_perm:[q,q,q,q]).
+template <int Q>
+__device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, Q * 0x55, 0xF, 0xF, true);
+}
+
+// fused GEMV on the matrix cores: v_mfma_f32_4x4x4_16b_bf16 multiplies, in each of its
+// 16 blocks, 4 rows x 4 k (operand A: lane 4*blk + row holds the 4 k values of that row)
+// by 4 k x 4 columns (operand B: lane 4*blk + col) into D[row][col] (register `row` of lane
+// 4*blk + col).  A lane's four pairs are exactly two A operands (columns 0..3 and 4..7 of
+// its row); lane 4*b + j supplies X[batch j] for those columns.  One accumulator set
+// covers batches 0..3, a second one batches 4..7.  Lanes whose batch does not exist
+// carry finite filler and their results are never stored.
+//
+// How X reaches the B operand depends on the batch:
+//   batch 1     the four lanes of a quad own the same 8 columns; each loads one X pair
+//               in the load phase (one register per step) and the quad shares them by DPP;
+//   batch 2..4  every lane loads its batch's 8 columns in the load phase (4 registers/step);
+//   batch 5..8  two sets would need 8 registers per step: X is fetched two steps ahead
+//               inside the compute phase instead (it is cache resident).
+template <int BS>
+struct MfmaPolicy {
+    static constexpr int NSET = BS <= 4 ? 1 : 2;
+    static constexpr bool QUARTER = BS == 1;
+    static constexpr bool PIPED = BS > 4;
+    static constexpr int XAHEAD = 2;
+    struct Slot { uint2 rem; uint4 x; };         // x: full columns (batch 2..4) or .x = own pair (batch 1)
+    struct Piped { uint4 x[NSET]; };
+    const uint2* rem0;
+    const uint4* x0[NSET];   // this lane's 8 X columns of the task's first step, per set
+    const uint32_t* xq0;     // batch 1: this lane's own X pair of the task's first step
+    int last;
+    uint4 xr[XAHEAD][NSET];
+    f32x4_t acc[NSET];
+
+    __device__ __forceinline__ void xload(uint4 (&dst)[NSET], int t) const {
+        t = t < last ? t : last;
+#pragma unroll
+        for (int q = 0; q < NSET; ++q) dst[q] = x0[q][(size_t)t * (kStepCols / 8)];
+    }
+    __device__ __forceinline__ void prime() {
+        if (PIPED) {
+#pragma unroll
+            for (int i = 0; i < XAHEAD; ++i) xload(xr[i], i);
+        }
+    }
+    __device__ __forceinline__ void load(Slot& s, int t) const {
+        t = t < last ? t : last;
+        s.rem = rem0[(size_t)t * kLanes];
+        if (QUARTER) s.x.x = xq0[(size_t)t * (kStepCols / 2)];
+        else if (!PIPED) s.x = x0[0][(size_t)t * (kStepCols / 8)];
+    }
+    __device__ __forceinline__ Piped take(const Slot& s, int i, int t) {
+        Piped p;
+        if (QUARTER) {
+            p.x[0] = make_uint4(s.x.x, quad_bcast<1>(s.x.x), quad_bcast<2>(s.x.x), quad_bcast<3>(s.x.x));
+        } else if (!PIPED) {
+            p.x[0] = s.x;
+        } else {
+#pragma unroll
+            for (int q = 0; q < NSET; ++q) p.x[q] = xr[i % XAHEAD][q];
+            xload(xr[i % XAHEAD], t + XAHEAD);
+        }
+        return p;
+    }
+    __device__ __forceinline__ void use(const Piped& s, int, const uint32_t (&w)[4]) {
+        const bf16x4_t a01 = __builtin_bit_cast(bf16x4_t, make_uint2(w[0], w[1]));
+        const bf16x4_t a23 = __builtin_bit_cast(bf16x4_t, make_uint2(w[2], w[3]));
+#pragma unroll
+        for (int q = 0; q < NSET; ++q) {
+            const bf16x4_t b01 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].x, s.x[q].y));
+            const bf16x4_t b23 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].z, s.x[q].w));
+            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a01, b01, acc[q], 0, 0, 0);
+            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a23, b23, acc[q], 0, 0, 0);
+        }
+    }
+};
+
+struct TaskId { int k, c, t0, t1; };
+
+__device__ __forceinline__ TaskId task_of(const Shape& s, int kc) {
+    TaskId id;
+    id.k = kc / s.nc;
+    id.c = kc % s.nc;
+    id.t0 = (s.steps * id.c) / s.nc;
+    id.t1 = (s.steps * (id.c + 1)) / s.nc;
+    return id;
+}
+
 // ------------------------------------------------------------------ decode to BF16
-__global__ __launch_bounds__(kBlockThreads)
+template <int NW>
+__global__ __launch_bounds__(NW * kLanes)
 void huffman_decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
                            uint16_t* __restrict__ Y, const uint32_t* __restrict__ offsets,
-                           const uint32_t* __restrict__ table, Shape s) {
+                           const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
     __shared__ uint32_t lut[kTableEntries];
+    __shared__ uint32_t rings[NW][kRingWords];
     load_table(lut, table);
     __syncthreads();
 
@@ -42,49 +187,38 @@ void huffman_decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __
     const int G = s.M / kGroupRows;
     const int per_group = s.split_k * s.nc;
     const long long ntasks = (long long)G * per_group;
-    long long task = (long long)blockIdx.x * kWavesPerBlock + wave;
+    const long long task = (long long)blockIdx.x * NW + wave;
     if (task >= ntasks) return;
     const int g = (int)(task / per_group);
-    const int kc = (int)(task % per_group);
-    const int k = kc / s.nc, c = kc % s.nc;
-    const int t0 = (s.steps * c) / s.nc, t1 = (s.steps * (c + 1)) / s.nc;
+    const TaskId id = task_of(s, (int)(task % per_group));
 
     HuffCursor cur;
-    cur.init(A_exp, task_span(offsets, s.M, s.split_k, s.nc, k, g, c, s.total_words), lane);
-
+    cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
     const int K = s.Ks * s.split_k;
-    const uint2* remp = (const uint2*)(A_rem + ((size_t)k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)t0 * kLanes + lane;
-    uint16_t* yp = Y + (size_t)(kGroupRows * g + (lane & 3)) * K + (size_t)k * s.Ks + (size_t)t0 * kStepCols + (lane >> 2) * kLaneCols;
-
-    uint2 r_next = remp[0];
-    for (int t = t0; t < t1; ++t) {
-        uint2 r = r_next;
-        remp += kLanes;
-        if (t + 1 < t1) r_next = remp[0];
-        uint32_t e[4];
-        cur.step(lut, e);
-        uint4 out;
-        out.x = rebuild_pair(e[0], rem_lo_pair(r.x));
-        out.y = rebuild_pair(e[1], rem_hi_pair(r.x));
-        out.z = rebuild_pair(e[2], rem_lo_pair(r.y));
-        out.w = rebuild_pair(e[3], rem_hi_pair(r.y));
-        *(uint4*)yp = out;
-        yp += kStepCols;
-    }
+    StorePolicy pol;
+    pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
+    pol.yp = Y + (size_t)(kGroupRows * g + (lane & 3)) * K + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols;
+    pol.last = id.t1 - id.t0 - 1;
+    if (header_has_esc(header)) run_task<true>(cur, lut, pol, id.t1 - id.t0);
+    else run_task<false>(cur, lut, pol, id.t1 - id.t0);
 }
 
 // ------------------------------------------------------------------ fused decode + GEMV
-// Block = 8 wavefronts.  The split_k*nc tasks of one row group are spread over
-// P = min(split_k*nc, 8) wavefronts of the same block (a wavefront loops when there
+// Block = NW wavefronts.  The split_k*nc tasks of one row group are spread over
+// P = min(split_k*nc, NW) wavefronts of the same block (a wavefront loops when there
 // are more tasks than that), so the sum over splits and chunks never leaves the block.
-template <int BS>
-__global__ __launch_bounds__(kBlockThreads)
+// register budget: at least this many wavefronts per SIMD must stay resident
+constexpr int min_waves(int bs) { return bs <= 1 ? 6 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
+
+template <int BS, int NW>
+__global__ __launch_bounds__(NW * kLanes)
 void gemv_huffman_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
                          const uint16_t* __restrict__ X, uint16_t* __restrict__ Y,
                          const uint32_t* __restrict__ offsets, const uint32_t* __restrict__ table,
-                         Shape s, int P, int groups_per_block) {
+                         const uint8_t* __restrict__ header, Shape s, int P, int groups_per_block) {
+    // The partial sums reuse the rings once every task of the block is done.
     __shared__ uint32_t lut[kTableEntries];
-    __shared__ float part[kWavesPerBlock][BS][kGroupRows];
+    __shared__ uint32_t rings[NW][kRingWords];
     load_table(lut, table);
     __syncthreads();
 
@@ -96,78 +230,72 @@ void gemv_huffman_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __re
     const int g = blockIdx.x * groups_per_block + rg;
     const bool active = rg < groups_per_block && g < G;
     const int K = s.Ks * s.split_k;
+    const bool has_esc = header_has_esc(header);
 
-    float acc[BS];
+    MfmaPolicy<BS> pol;
+    constexpr int NSET = MfmaPolicy<BS>::NSET;
 #pragma unroll
-    for (int b = 0; b < BS; ++b) acc[b] = 0.f;
+    for (int q = 0; q < NSET; ++q) pol.acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     if (active) {
         for (int kc = p; kc < per_group; kc += P) {
-            const int k = kc / s.nc, c = kc % s.nc;
-            const int t0 = (s.steps * c) / s.nc, t1 = (s.steps * (c + 1)) / s.nc;
+            const TaskId id = task_of(s, kc);
             HuffCursor cur;
-            cur.init(A_exp, task_span(offsets, s.M, s.split_k, s.nc, k, g, c, s.total_words), lane);
-            const uint2* remp = (const uint2*)(A_rem + ((size_t)k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)t0 * kLanes + lane;
-            const uint16_t* xp = X + (size_t)k * s.Ks + (size_t)t0 * kStepCols + (lane >> 2) * kLaneCols;
-
-            uint2 r_next = remp[0];
-            uint4 x_next[BS];
+            cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
+            pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
 #pragma unroll
-            for (int b = 0; b < BS; ++b) x_next[b] = *(const uint4*)(xp + (size_t)b * K);
-            for (int t = t0; t < t1; ++t) {
-                uint2 r = r_next;
-                uint4 x[BS];
+            for (int q = 0; q < NSET; ++q) {
+                const int batch = (lane & 3) + 4 * q;
+                pol.x0[q] = (const uint4*)(X + (size_t)(batch < BS ? batch : 0) * K + (size_t)id.k * s.Ks
+                                           + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols);
+            }
+            pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
+            pol.last = id.t1 - id.t0 - 1;
+            if (has_esc) run_task<true>(cur, lut, pol, id.t1 - id.t0);
+            else run_task<false>(cur, lut, pol, id.t1 - id.t0);
+        }
+        // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
 #pragma unroll
-                for (int b = 0; b < BS; ++b) x[b] = x_next[b];
-                remp += kLanes;
-                xp += kStepCols;
-                if (t + 1 < t1) {
-                    r_next = remp[0];
+        for (int q = 0; q < NSET; ++q) {
 #pragma unroll
-                    for (int b = 0; b < BS; ++b) x_next[b] = *(const uint4*)(xp + (size_t)b * K);
-                }
-                uint32_t e[4];
-                cur.step(lut, e);
-                const uint32_t w0 = rebuild_pair(e[0], rem_lo_pair(r.x));
-                const uint32_t w1 = rebuild_pair(e[1], rem_hi_pair(r.x));
-                const uint32_t w2 = rebuild_pair(e[2], rem_lo_pair(r.y));
-                const uint32_t w3 = rebuild_pair(e[3], rem_hi_pair(r.y));
-#pragma unroll
-                for (int b = 0; b < BS; ++b) {
-                    float a = acc[b];
-                    a = dot2(w0, x[b].x, a);
-                    a = dot2(w1, x[b].y, a);
-                    a = dot2(w2, x[b].z, a);
-                    a = dot2(w3, x[b].w, a);
-                    acc[b] = a;
-                }
+            for (int i = 0; i < kGroupRows; ++i) {
+                float a = pol.acc[q][i];
+                a += __shfl_xor(a, 4);
+                a += __shfl_xor(a, 8);
+                a += __shfl_xor(a, 16);
+                a += __shfl_xor(a, 32);
+                pol.acc[q][i] = a;
             }
         }
-        // lanes 4*b + i hold partial sums of row i: fold the 16 column blocks
+    }
+    __syncthreads();                       // every wavefront has finished reading its ring
+    float* mine = (float*)rings[wave];     // partial sums: [set][row][batch lane]
+    if (active && lane < 4) {
 #pragma unroll
-        for (int b = 0; b < BS; ++b) {
-            float a = acc[b];
-            a += __shfl_xor(a, 4);
-            a += __shfl_xor(a, 8);
-            a += __shfl_xor(a, 16);
-            a += __shfl_xor(a, 32);
-            if (lane < kGroupRows) part[wave][b][lane] = a;
-        }
+        for (int q = 0; q < NSET; ++q)
+#pragma unroll
+            for (int i = 0; i < kGroupRows; ++i) mine[(q * kGroupRows + i) * 4 + lane] = pol.acc[q][i];
     }
     __syncthreads();
-    if (active && p == 0 && lane < kGroupRows) {
+    if (active && p == 0 && lane < 4) {
 #pragma unroll
-        for (int b = 0; b < BS; ++b) {
-            float a = 0.f;
-            for (int q = 0; q < P; ++q) a += part[rg * P + q][b][lane];
-            Y[(size_t)b * s.M + kGroupRows * g + lane] = f32_to_bf16_rne(a);
+        for (int q = 0; q < NSET; ++q) {
+            const int batch = lane + 4 * q;
+            if (batch < BS) {
+#pragma unroll
+                for (int i = 0; i < kGroupRows; ++i) {
+                    float a = 0.f;
+                    for (int w = 0; w < P; ++w) a += ((const float*)rings[rg * P + w])[(q * kGroupRows + i) * 4 + lane];
+                    Y[(size_t)batch * s.M + kGroupRows * g + i] = f32_to_bf16_rne(a);
+                }
+            }
         }
     }
 }
 
 // ------------------------------------------------------------------ encoder
-// One wavefront per task; it replays the decoder's refill schedule and writes each
-// finished word at the stream position the decoder will read it from.
+// One wavefront per task: every lane packs its own codes into its own column of the
+// task block; the block gets as many rows as the longest lane needs.
 __global__ __launch_bounds__(kLanes)
 void huffman_encode_kernel(const uint8_t* __restrict__ data, const uint32_t* __restrict__ enc,
                            uint32_t* __restrict__ output, uint32_t* __restrict__ output_lengths,
@@ -191,26 +319,20 @@ void huffman_encode_kernel(const uint8_t* __restrict__ data, const uint32_t* __r
             bits += en >> 16;
         }
     }
-    const uint32_t nwords = (bits + 31u) >> 5;
-    const uint32_t nref = nwords > (uint32_t)kInitWords ? nwords - kInitWords : 0u;
-    uint32_t sum_ref = nref, sum_esc = nesc;
+    uint32_t rows = (bits + 31u) >> 5, sum_esc = nesc;
     for (int o = 32; o > 0; o >>= 1) {
-        sum_ref += __shfl_xor(sum_ref, o);
+        uint32_t r2 = __shfl_xor(rows, o);
+        rows = r2 > rows ? r2 : rows;
         sum_esc += __shfl_xor(sum_esc, o);
     }
-    const uint32_t body = kInitWords * kLanes + sum_ref + sum_esc;
+    const uint32_t body = rows * kLanes + sum_esc;
     const uint32_t total = (body + kAlignWords - 1) / kAlignWords * kAlignWords;
     if (lane == 0) output_lengths[task] = total;
-    // zero padding between refill words and escape list
-    for (uint32_t i = kInitWords * kLanes + sum_ref + lane; i < total - sum_esc; i += kLanes) out[i] = 0;
+    for (uint32_t i = body + lane; i < total; i += kLanes) out[i] = 0;
 
-    // pass 2: emit.  a0/a1 hold the bits of words m, m+1, m+2 (m = cursor word).
-    uint64_t a0 = nref;
-    uint32_t a1 = 0;
-    uint32_t fill = kHeaderBits;                 // bit position relative to word m
-    uint32_t q0 = lane, q1 = kLanes + lane, q2 = 2 * kLanes + lane;   // stream slots of words m, m+1, m+2
-    const uint32_t kNone = 0xFFFFFFFFu;
-    uint32_t left = nref, ptr = kInitWords * kLanes, eptr = 0;
+    // pass 2: emit
+    uint64_t acc = 0;
+    uint32_t fill = kHeaderBits, row = 0, eptr = 0;
     for (int t = 0; t < n_steps; ++t) {
         uint2 d = dp[(size_t)t * kLanes];
         uint32_t pr[4] = {d.x & 0xFFFFu, d.x >> 16, d.y & 0xFFFFu, d.y >> 16};
@@ -224,35 +346,20 @@ void huffman_encode_kernel(const uint8_t* __restrict__ data, const uint32_t* __r
                 out[total - 1 - (eptr + lane_rank(m))] = pr[q];
             }
             eptr += (uint32_t)__builtin_popcountll(m);
-            const uint32_t code = en & 0xFFFFu, len = en >> 16;
-            if (fill < 64u) {
-                a0 |= (uint64_t)code << fill;
-                if (fill + len > 64u) a1 |= code >> (64u - fill);
-            } else {
-                a1 |= code << (fill - 64u);
-            }
-            fill += len;
-        }
-        for (;;) {
-            bool cross = fill >= 32u + kCursorBias;
-            if (ballot(cross) == 0) break;
-            bool load = cross && left != 0;
-            uint64_t m = ballot(load);
-            if (cross) {
-                if (q0 != kNone) out[q0] = (uint32_t)a0;
-                a0 = (a0 >> 32) | ((uint64_t)a1 << 32);
-                a1 = 0;
+            acc |= (uint64_t)(en & 0xFFFFu) << fill;          // fill < 32, code <= 12 bits
+            fill += en >> 16;
+            if (fill >= 32u) {
+                out[(size_t)row * kLanes + lane] = (uint32_t)acc;
+                acc >>= 32;
                 fill -= 32u;
-                q0 = q1; q1 = q2;
-                q2 = load ? ptr + lane_rank(m) : kNone;
-                if (load) left -= 1;
+                row++;
             }
-            ptr += (uint32_t)__builtin_popcountll(m);
         }
     }
-    if (q0 != kNone) out[q0] = (uint32_t)a0;
-    if (q1 != kNone) out[q1] = (uint32_t)(a0 >> 32);
-    if (q2 != kNone) out[q2] = a1;
+    for (; row < rows; ++row) {
+        out[(size_t)row * kLanes + lane] = (uint32_t)acc;
+        acc >>= 32;
+    }
 }
 
 }  // namespace bhi
@@ -278,61 +385,71 @@ static int check_shape(int split_k, int M, int Ks, int64_t exp_words, int64_t lu
 extern "C" int bhi_huffman_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
                                   void* Y, const void* offsets,
                                   const void* LUT1, int64_t lut1_bytes,
-                                  const void*, const void*, const void*, const void*,
+                                  const void*, const void*, const void*, const void* code_lengths,
                                   int split_k, int M, int Ks, void* stream) {
-    if (!A_rem || !A_exp || !Y || !offsets || !LUT1) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (!A_rem || !A_exp || !Y || !offsets || !LUT1 || !code_lengths) return bhi_fail(BHI_EINVAL, "null pointer");
     Shape s;
     if (int rc = check_shape(split_k, M, Ks, exp_words, lut1_bytes, &s)) return rc;
+    constexpr int NW = 4;
     long long ntasks = (long long)(M / kGroupRows) * split_k * s.nc;
-    unsigned grid = (unsigned)((ntasks + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL(huffman_decode_kernel, dim3(grid), dim3(kBlockThreads), 0, (hipStream_t)stream,
+    unsigned grid = (unsigned)((ntasks + NW - 1) / NW);
+    hipLaunchKernelGGL(huffman_decode_kernel<NW>, dim3(grid), dim3(NW * kLanes), 0, (hipStream_t)stream,
                        (const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
-                       (const uint32_t*)LUT1, s);
+                       (const uint32_t*)LUT1, (const uint8_t*)code_lengths, s);
     return bhi_launch_status("huffman_decode");
 }
 
 template <int BS>
 static void launch_gemv(const void* A_rem, const void* A_exp, const void* X, void* Y, const void* offsets,
-                        const void* LUT1, const Shape& s, hipStream_t stream) {
-    int per_group = s.split_k * s.nc;
-    int P = per_group < kWavesPerBlock ? per_group : kWavesPerBlock;
-    int gpb = kWavesPerBlock / P;
-    int G = s.M / kGroupRows;
-    unsigned grid = (unsigned)((G + gpb - 1) / gpb);
-    hipLaunchKernelGGL(gemv_huffman_kernel<BS>, dim3(grid), dim3(kBlockThreads), 0, stream,
-                       (const uint8_t*)A_rem, (const uint32_t*)A_exp, (const uint16_t*)X, (uint16_t*)Y,
-                       (const uint32_t*)offsets, (const uint32_t*)LUT1, s, P, gpb);
+                        const void* LUT1, const void* header, const Shape& s, hipStream_t stream) {
+    const int per_group = s.split_k * s.nc;
+    const int G = s.M / kGroupRows;
+    // small blocks spread more evenly over the 256 CUs; 8 wavefronts only when one row
+    // group needs more than 4 of them
+    if (per_group <= 4) {
+        constexpr int NW = 4;
+        const int P = per_group, gpb = NW / P;
+        hipLaunchKernelGGL((gemv_huffman_kernel<BS, NW>), dim3((unsigned)((G + gpb - 1) / gpb)), dim3(NW * kLanes), 0, stream,
+                           (const uint8_t*)A_rem, (const uint32_t*)A_exp, (const uint16_t*)X, (uint16_t*)Y,
+                           (const uint32_t*)offsets, (const uint32_t*)LUT1, (const uint8_t*)header, s, P, gpb);
+    } else {
+        constexpr int NW = 8;
+        const int P = per_group < NW ? per_group : NW, gpb = NW / P;
+        hipLaunchKernelGGL((gemv_huffman_kernel<BS, NW>), dim3((unsigned)((G + gpb - 1) / gpb)), dim3(NW * kLanes), 0, stream,
+                           (const uint8_t*)A_rem, (const uint32_t*)A_exp, (const uint16_t*)X, (uint16_t*)Y,
+                           (const uint32_t*)offsets, (const uint32_t*)LUT1, (const uint8_t*)header, s, P, gpb);
+    }
 }
 
 extern "C" int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64_t exp_words,
                                      const void* X, void* Y, const void* offsets,
                                      const void* LUT1, int64_t lut1_bytes,
-                                     const void*, const void*, const void*, const void*,
+                                     const void*, const void*, const void*, const void* code_lengths,
                                      int split_k, int M, int Ks, int batch, void* stream) {
-    if (!A_rem || !A_exp || !X || !Y || !offsets || !LUT1) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (!A_rem || !A_exp || !X || !Y || !offsets || !LUT1 || !code_lengths) return bhi_fail(BHI_EINVAL, "null pointer");
     if (batch < 1) return bhi_fail(BHI_EINVAL, "batch must be >= 1");
     if (batch > kMaxBatch) return bhi_fail(BHI_EBATCH, "fused GEMV supports batch <= 8");
     Shape s;
     if (int rc = check_shape(split_k, M, Ks, exp_words, lut1_bytes, &s)) return rc;
     hipStream_t st = (hipStream_t)stream;
     switch (batch) {
-        case 1: launch_gemv<1>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        case 2: launch_gemv<2>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        case 3: launch_gemv<3>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        case 4: launch_gemv<4>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        case 5: launch_gemv<5>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        case 6: launch_gemv<6>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        case 7: launch_gemv<7>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
-        default: launch_gemv<8>(A_rem, A_exp, X, Y, offsets, LUT1, s, st); break;
+        case 1: launch_gemv<1>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        case 2: launch_gemv<2>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        case 3: launch_gemv<3>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        case 4: launch_gemv<4>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        case 5: launch_gemv<5>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        case 6: launch_gemv<6>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        case 7: launch_gemv<7>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
+        default: launch_gemv<8>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
     }
     return bhi_launch_status("gemv_bf16_huffman");
 }
 
 extern "C" int64_t bhi_encode_capacity(int n_steps) {
     if (n_steps < 1) return 0;
-    // init words + every lane full of 12-bit codes + every pair escaped + alignment
+    // every lane full of 12-bit codes + every pair escaped + alignment
     int64_t lane_words = ((int64_t)kHeaderBits + (int64_t)n_steps * kPairsPerStep * kTableBits + 31) / 32;
-    return kInitWords * kLanes + (int64_t)kLanes * lane_words + (int64_t)n_steps * kPairsPerStep * kLanes + kAlignWords;
+    return (int64_t)kLanes * lane_words + (int64_t)n_steps * kPairsPerStep * kLanes + kAlignWords;
 }
 
 extern "C" int bhi_huffman_encode(const void* data, const void* LUT, void* output, void* output_lengths,

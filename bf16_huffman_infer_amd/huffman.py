@@ -19,7 +19,7 @@ import numpy as np
 import torch
 
 TABLE_BITS = 12
-ESC_FLAG = 0x80
+ESC_FLAG = 1 << 15
 ESC_INDEX = 65536
 ESC_SIDE_BITS = 32            # one stream word per escaped pair
 MAX_CODED = 3072              # never give more than this many pairs a code of their own
@@ -74,11 +74,13 @@ class LUTHuffmanEncoder:
 
     * ``enc_table``  uint32 ``[65537]``: ``code | len<<16`` per pair (0 = escaped), ESC in
       slot 65536; code bits are emitted LSB first.
-    * ``dec_table``  uint32 ``[4096]``: ``a | b<<16 | len<<24`` (``|0x80<<24`` for ESC).
+    * ``dec_table``  uint32 ``[4096]``: ``len | a<<7 | b<<23`` (``| 1<<15`` for ESC): the two
+      exponents already sit at their BF16 bit positions of a packed pair.
     * ``LUT1``       the decode table viewed as uint8 ``[16384]`` -- the module buffer.
     * ``LUT2..LUT4`` uint8 ``[256]`` filled with 255: the reference's deeper cascade
       levels have no job when no code is longer than the first-level window.
-    * ``code_lengths`` uint8 ``[256]``: a format header (version, table bits, ESC length).
+    * ``code_lengths`` uint8 ``[256]``: a format header (version, table bits, ESC length,
+      whether any pair of the histogram is escaped).
     """
 
     def __init__(self, max_code_length: int = TABLE_BITS):
@@ -153,9 +155,9 @@ class LUTHuffmanEncoder:
             self.enc_table[sym] = rev | (ln << 16)
             idx = rev + (np.arange(1 << (TABLE_BITS - ln)) << ln)
             if sym == ESC_INDEX:
-                self.dec_table[idx] = (ln | ESC_FLAG) << 24
+                self.dec_table[idx] = ln | ESC_FLAG
             else:
-                self.dec_table[idx] = (sym & 0xFF) | ((sym >> 8) << 16) | (ln << 24)
+                self.dec_table[idx] = ln | ((sym & 0xFF) << 7) | ((sym >> 8) << 23)
             filled[idx] = True
             code += 1
         assert filled.all() and code == (1 << prev_len), "code is not complete"
@@ -164,3 +166,4 @@ class LUTHuffmanEncoder:
         self.code_lengths[0] = 1                      # format version
         self.code_lengths[1] = TABLE_BITS
         self.code_lengths[2] = int(self.enc_table[ESC_INDEX]) >> 16
+        self.code_lengths[3] = 1 if int(counts.sum() - counts[coded].sum()) > 0 else 0   # escapes occur

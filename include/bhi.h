@@ -37,8 +37,8 @@ extern "C" {
  * (the reference duplicates OP_PER_LANE / ANS_PRECISION in functional.py:15-16 and
  * kernel.cu:22-25).  Fills out[0..n) with, in order:
  *   0 format version        1 lanes per wavefront (64)   2 rows per row group (4)
- *   3 columns per step (128)4 Huffman table index bits   5 init words per lane (3)
- *   6 header bits per lane  7 max fused batch            8 rANS precision bits
+ *   3 columns per step (128)4 Huffman table index bits   5 window words per lane (3)
+ *   6 dummy bits per lane   7 max fused batch            8 rANS precision bits
  *   9 stream alignment in 32-bit words                   10 tail padding words
  *  11 task target used by bhi_chunks_per_group           12 max steps per task
  * Returns the number of constants available. */
@@ -58,7 +58,8 @@ const char* bhi_last_error_string(void);
  *   Y       bf16   [batch, M]        written
  *   offsets int32  [split_k, M]
  *   LUT1    uint8  [lut1_bytes]      pair decode table, lut1_bytes = 4 << table bits
- *   LUT2..4, code_lengths uint8 [256] (carried for the op signature; not read) */
+ *   LUT2..4 uint8 [256] (carried for the op signature; not read)
+ *   code_lengths uint8 [256]        format header: version, table bits, ESC length, has-escapes */
 int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64_t exp_words,
                           const void* X, void* Y, const void* offsets,
                           const void* LUT1, int64_t lut1_bytes,

@@ -19,22 +19,21 @@ rem plane   uint8 ``[split_k, M, Ks]``; the ``4*Ks`` bytes of (k, g) hold step `
 code        one length-limited (<= 12 bit) Huffman code over exponent *pairs*
             ``a | b<<8`` (a = even column) plus an ESC word; code bits are consumed
             LSB first.  ``dec`` is the 4096-entry decode table indexed by the next 12
-            stream bits: ``a | b<<16 | len<<24``; ESC entries carry ``0x80`` in the top
-            byte beside the length.  The two raw exponents of an escaped pair are
-            not in the bitstream: they sit in the task's escape list.
-lane bits   bits 0..7 of a lane's bitstring = number of refill loads the lane will
-            make; codes follow from bit 8.  The bitstring is cut into 32-bit words.
-task stream ``[192 init words][refill words][zero pad][escape list]``, a multiple of 4
-            words.  Init: word ``n`` (n < 3) of lane ``l`` at ``64*n + l``.  Refill words
-            are stored in the order the decoder consumes them: after every step,
-            while any lane's cursor has left its current word, each such lane
-            advances one word and -- if it still has refill loads left -- takes the
-            next stream word, lanes in ascending order (a ballot prefix count).  The
-            cursor is ``bit position - 2`` (the decoder keeps its window shifted left
-            by two so that ``window & 0x3FFC`` is the byte address of the table entry),
-            so a lane leaves word ``m`` when ``position - 2 >= 32*(m+1)``.
-            Escape entries ``a | b<<8`` are consumed per step in (pair, lane) order and
-            stored backwards from the end of the task stream.
+            stream bits: ``len | a<<7 | b<<23`` (the exponents sit where a packed BF16
+            pair needs them); ESC entries are ``len | 1<<15``.  The two raw exponents
+            of an escaped pair are not in the bitstream: they sit in the task's
+            escape list.
+lane bits   a lane's codes are concatenated from bit 2 of its private bitstring (the
+            decoder keeps its window shifted left by two so that ``window & 0x3FFC`` is
+            the byte address of the table entry) and the bitstring is cut into
+            32-bit words.
+task block  ``[W rows of 64 words][escape list][zero pad]``, a multiple of 4 words:
+            word ``w`` of lane ``l`` sits at ``64*w + l`` and ``W`` is the longest lane of
+            the task (shorter lanes are zero padded).  Lanes at different depths
+            read different rows, but row ``w`` of lane ``l`` always falls into LDS bank
+            ``l mod 32``: the per-step window reads are conflict free.  Escape entries
+            ``a | b<<8`` are consumed per step in (pair, lane) order and stored
+            backwards from the end of the task block.
 offsets     int32 ``[split_k, M]``: word offset of task (k, g, c) at ``[k, 4*g + c]``;
             tasks are laid out in (k, g, c) order; unused slots are 0.
 
@@ -52,16 +51,15 @@ GROUP_ROWS = 4
 LANE_COLS = 8
 STEP_COLS = 128
 PAIRS_PER_STEP = 4
-INIT_WORDS = 3
-HEADER_BITS = 8
+WINDOW_WORDS = 3           # words of its bitstring a lane looks at per step
+HEADER_BITS = 2            # dummy bits in front of every lane's codes
 TABLE_BITS = 12
-ESC_FLAG = 0x80
-CURSOR_BIAS = 2            # the decoder's cursor trails the bit position by 2 (pre-shifted window)
+ESC_FLAG = 1 << 15
 TARGET_TASKS = 4096
 MIN_CHUNK_STEPS = 4
 MAX_CHUNKS = 4
 ALIGN_WORDS = 4
-TAIL_PAD_WORDS = 1024
+TAIL_PAD_WORDS = 2048
 ESC_INDEX = 65536          # slot of the ESC code in the encoder table
 
 
@@ -127,50 +125,24 @@ def _encode_tasks(sym: np.ndarray, enc: np.ndarray):
     code_l = code.transpose(0, 2, 1, 3).reshape(nt, LANES, ns * PAIRS_PER_STEP)
     end = HEADER_BITS + np.cumsum(ln_l, axis=-1)
     off = end - ln_l
-    total_bits = end[..., -1]
-    nwords = (total_bits + 31) // 32
-    nref = np.maximum(nwords - INIT_WORDS, 0)
-    assert nref.max() <= 255
-    maxw = max(int(nwords.max()), INIT_WORDS) + 1
-    lw = np.zeros((nt, LANES, maxw), dtype=np.uint64)
+    nwords = (end[..., -1] + 31) // 32                               # [nt, 64]
+    rows = nwords.max(axis=-1)                                       # [nt]
+    lw = np.zeros((nt, LANES, int(rows.max()) + 1), dtype=np.uint64)
     ti, li, _ = np.indices(off.shape)
     val = code_l << (off & 31).astype(np.uint64)
     np.bitwise_or.at(lw, (ti, li, off >> 5), val & np.uint64(0xFFFFFFFF))
     np.bitwise_or.at(lw, (ti, li, (off >> 5) + 1), val >> np.uint64(32))
-    lw[..., 0] |= nref.astype(np.uint64)
-
-    # refill schedule: cursor word after each step
-    step_bits = ln.sum(axis=-1).transpose(0, 2, 1)                   # [nt, 64, ns]
-    cur = (HEADER_BITS - CURSOR_BIAS + np.cumsum(step_bits, axis=-1)) >> 5   # cursor word after step t
-    prev = np.concatenate([np.zeros((nt, LANES, 1), np.int64), cur[..., :-1]], axis=-1)
-    cross = cur - prev
-    assert cross.max() <= 2
-    loads = np.zeros((nt, ns, 2, LANES), dtype=bool)
-    widx = np.zeros((nt, ns, 2, LANES), dtype=np.int64)
-    for r in range(2):
-        ordinal = prev + r + 1                                       # 1-based crossing number
-        do = (cross > r) & (ordinal <= nref[..., None])
-        loads[:, :, r, :] = do.transpose(0, 2, 1)
-        widx[:, :, r, :] = (ordinal + INIT_WORDS - 1).transpose(0, 2, 1)
-    flat = loads.reshape(nt, -1)
-    pos = np.cumsum(flat, axis=-1) - flat                            # exclusive rank
-    nrefill = flat.sum(axis=-1)
-    assert np.array_equal(nrefill, nref.sum(axis=-1))
 
     esc_flat = esc.transpose(0, 1, 3, 2).reshape(nt, -1)             # (step, pair, lane) order
     pair_flat = pairs.transpose(0, 1, 3, 2).reshape(nt, -1)
     nesc = esc_flat.sum(axis=-1)
 
     streams = []
-    lane_of = np.broadcast_to(np.arange(LANES), (ns, 2, LANES)).reshape(-1)
     for t in range(nt):
-        body = INIT_WORDS * LANES + int(nrefill[t]) + int(nesc[t])
+        body = int(rows[t]) * LANES + int(nesc[t])
         total = (body + ALIGN_WORDS - 1) // ALIGN_WORDS * ALIGN_WORDS
         st = np.zeros(total, dtype=np.uint32)
-        for n in range(INIT_WORDS):
-            st[n * LANES:(n + 1) * LANES] = lw[t, :, n].astype(np.uint32)
-        sel = flat[t]
-        st[INIT_WORDS * LANES + pos[t][sel]] = lw[t, lane_of[sel], widx[t].reshape(-1)[sel]].astype(np.uint32)
+        st[:int(rows[t]) * LANES] = lw[t, :, :int(rows[t])].T.reshape(-1).astype(np.uint32)
         if nesc[t]:
             st[total - 1 - np.arange(int(nesc[t]))] = pair_flat[t][esc_flat[t]]
         streams.append(st)
@@ -215,35 +187,32 @@ def encode(bits: np.ndarray, split_k: int, enc: np.ndarray):
 def _decode_tasks(words: np.ndarray, base: np.ndarray, end: np.ndarray, ns: int, dec: np.ndarray) -> np.ndarray:
     """Step-by-step model of one wavefront per task.
 
-    words: uint32 flat buffer; base/end: [nt] word offsets of each task stream and of
-    the stream that follows it.  Returns uint8 [nt, ns, 64, 8].
+    words: uint32 flat buffer; base/end: [nt] word offsets of each task block and of
+    the block that follows it.  Returns uint8 [nt, ns, 64, 8].
     """
     nt = len(base)
     U = np.uint64
     lanes = np.arange(LANES)
     w64 = words.astype(np.uint64)
-    lo = w64[base[:, None] + lanes]
-    hi = w64[base[:, None] + LANES + lanes]
-    nx = w64[base[:, None] + 2 * LANES + lanes]
-    left = (lo & U(0xFF)).astype(np.int64)
-    c = np.full((nt, LANES), HEADER_BITS - CURSOR_BIAS, dtype=np.int64)
-    ptr = np.zeros(nt, dtype=np.int64)
+    pos = np.zeros((nt, LANES), dtype=np.int64)        # cursor = bit position - 2 (the window is pre-shifted)
     eptr = np.zeros(nt, dtype=np.int64)
     out = np.zeros((nt, ns, LANES, LANE_COLS), dtype=np.uint8)
     dec64 = dec.astype(np.uint64)
     M32 = U(0xFFFFFFFF)
     for t in range(ns):
-        cu = c.astype(np.uint64)
+        row = pos >> 5
+        at = base[:, None] + row * LANES + lanes
+        lo, hi, nx = w64[at], w64[at + LANES], w64[at + 2 * LANES]
+        cu = (pos & 31).astype(np.uint64)
         wlo = (((hi << U(32)) | lo) >> cu) & M32
         whi = (((nx << U(32)) | hi) >> cu) & M32
         win = (whi << U(32)) | wlo
-        used = np.zeros((nt, LANES), dtype=np.int64)
         for q in range(PAIRS_PER_STEP):
-            e = dec64[((win >> U(CURSOR_BIAS)) & U((1 << TABLE_BITS) - 1)).astype(np.int64)]
-            ln = ((e >> U(24)) & U(0x7F)).astype(np.int64)
-            esc = ((e >> U(31)) & U(1)).astype(bool)
-            a = (e & U(0xFF)).astype(np.uint8)
-            b = ((e >> U(16)) & U(0xFF)).astype(np.uint8)
+            e = dec64[((win >> U(HEADER_BITS)) & U((1 << TABLE_BITS) - 1)).astype(np.int64)]
+            ln = (e & U(0x1F)).astype(np.int64)
+            esc = ((e >> U(15)) & U(1)).astype(bool)
+            a = ((e >> U(7)) & U(0xFF)).astype(np.uint8)
+            b = ((e >> U(23)) & U(0xFF)).astype(np.uint8)
             if esc.any():
                 rank = np.cumsum(esc, axis=-1) - esc
                 src = end[:, None] - 1 - (eptr[:, None] + rank)
@@ -254,21 +223,7 @@ def _decode_tasks(words: np.ndarray, base: np.ndarray, end: np.ndarray, ns: int,
             out[:, t, :, 2 * q] = a
             out[:, t, :, 2 * q + 1] = b
             win = win >> ln.astype(np.uint64)
-            used += ln
-        c += used
-        assert c.max() < 96
-        while (c >= 32).any():
-            cross = c >= 32
-            c = np.where(cross, c - 32, c)
-            lo = np.where(cross, hi, lo)
-            hi = np.where(cross, nx, hi)
-            load = cross & (left > 0)
-            rank = np.cumsum(load, axis=-1) - load
-            src = base[:, None] + INIT_WORDS * LANES + ptr[:, None] + rank
-            nx = np.where(load, w64[np.where(load, src, 0)], nx)
-            left -= load
-            ptr += load.sum(axis=-1)
-    assert (left == 0).all()
+            pos = pos + ln
     return out
 
 
@@ -313,9 +268,9 @@ def check_tables(dec: np.ndarray, enc: np.ndarray) -> None:
         covered[idx] += 1
         got = dec[idx]
         if p == ESC_INDEX:
-            assert (got >> 24 == (ln | ESC_FLAG)).all()
+            assert (got == (ln | ESC_FLAG)).all()
         else:
-            want = (p & 0xFF) | ((p >> 8) << 16) | (ln << 24)
+            want = ln | ((p & 0xFF) << 7) | ((p >> 8) << 23)
             assert (got == want).all(), (p, ln)
     assert (covered == 1).all()
     assert abs(kraft - 1.0) < 1e-9

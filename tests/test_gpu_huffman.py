@@ -25,7 +25,7 @@ def _compress(w, n=None):
 
 
 @pytest.mark.parametrize("kind,M,K,n", [
-    ("gauss", 128, 384, None), ("gauss", 256, 512, 2), ("t3", 128, 1024, None), ("bits", 128, 256, None),
+    ("gauss", 128, 384, None), ("gauss", 256, 512, 2), ("t3", 128, 1024, None), ("bits", 128, 384, None),
     ("special", 256, 1280, None), ("zeros", 128, 128 * 3, None), ("gauss", 1024, 4096, None),
     ("gauss", 128, 2048, 4),
 ])
@@ -56,7 +56,7 @@ def test_encoder_matches_oracle_and_decodes(cuda, kind, M, K, n):
 
 
 @pytest.mark.parametrize("bs", [1, 2, 3, 4, 5, 6, 7, 8])
-@pytest.mark.parametrize("kind,M,K,n", [("gauss", 256, 1024, None), ("t3", 128, 512, 2), ("bits", 128, 256, None)])
+@pytest.mark.parametrize("kind,M,K,n", [("gauss", 256, 1024, None), ("t3", 128, 512, 2), ("bits", 128, 384, None)])
 def test_fused_gemv_matches_fp32(cuda, kind, M, K, n, bs):
     w = MAKERS[kind](M, K, seed=5)
     if kind == "bits":                      # keep the reference product finite
@@ -74,7 +74,7 @@ def test_large_batch_falls_back_to_decode_then_gemm(cuda):
     from bf16_huffman_infer_amd.functional import CompressedLinear
     w = gaussian_weight(256, 512, seed=7)
     bias = torch.randn(256).bfloat16()
-    lin = CompressedLinear(_compress(w), bias).cuda()
+    lin = CompressedLinear(_compress(w), torch.nn.Parameter(bias, requires_grad=False)).cuda()
     x = torch.randn(3, 5, 512).bfloat16().cuda()            # 15 rows > 8
     y = lin(x)
     ref = torch.nn.functional.linear(x, w.cuda(), bias.cuda())
@@ -86,12 +86,12 @@ def test_large_batch_falls_back_to_decode_then_gemm(cuda):
 
 def test_ops_reject_cpu_tensors_and_big_batch(cuda):
     from bf16_huffman_infer_amd import ops
-    mod = _compress(gaussian_weight(128, 256, seed=1))
-    y = torch.empty(128, 256, dtype=torch.bfloat16)
+    mod = _compress(gaussian_weight(128, 384, seed=1))
+    y = torch.empty(128, 384, dtype=torch.bfloat16)
     with pytest.raises((RuntimeError, NotImplementedError)):
         ops.huffman_decode(mod.rem, mod.exp, y, mod.offsets, mod.LUT1, mod.LUT2, mod.LUT3, mod.LUT4, mod.code_lengths)
     mod = mod.cuda()
-    x = torch.zeros(9, 1, 256, dtype=torch.bfloat16, device="cuda")
+    x = torch.zeros(9, 1, 384, dtype=torch.bfloat16, device="cuda")
     out = torch.empty(9, 128, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(RuntimeError, match="batch"):
         ops.gemv_bf16_huffman(mod.rem, mod.exp, x, out, mod.offsets, mod.LUT1, mod.LUT2, mod.LUT3, mod.LUT4,

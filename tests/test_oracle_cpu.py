@@ -1,0 +1,257 @@
+"""CPU checks that pin the oracle and the host-side logic (no GPU needed)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (bits_of, gaussian_weight, pair_counts, random_bits_weight, special_values_weight,
+                     student_t_weight)
+from oracle import planes, ref_layout, ref_tables, wave64
+
+
+# ----------------------------------------------------------------------------- bit planes
+def test_split_rebuild_all_65536_patterns():
+    bits = np.arange(65536, dtype=np.uint16)
+    rem, exp = planes.split_bf16(bits)
+    assert np.array_equal(planes.rebuild_bf16(rem, exp), bits)
+    # field positions against IEEE bfloat16: sign 15, exponent 14..7, mantissa 6..0
+    f = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).float()
+    m, e = torch.frexp(f[(exp > 0) & (exp < 255)])
+    assert np.array_equal((e.numpy() + 126).astype(np.uint8), exp[(exp > 0) & (exp < 255)])
+    assert np.array_equal((rem >> 7).astype(bool), (bits >> 15).astype(bool))
+    assert np.array_equal(rem & 0x7F, (bits & 0x7F).astype(np.uint8))
+
+
+def test_product_split_matches_oracle():
+    from bf16_huffman_infer_amd.utils import split_bf16
+    w = special_values_weight(64, 128, seed=2)
+    rem, exp = split_bf16(w)
+    orem, oexp = planes.split_bf16(bits_of(w))
+    assert np.array_equal(rem.numpy(), orem) and np.array_equal(exp.numpy(), oexp)
+
+
+@pytest.mark.parametrize("n,want", [(4096, 1), (3584, 1), (12288, 3), (18944, 4), (11008, 2), (384, 1),
+                                    (8192, 2), (5120, 2), (14336, 4), (28672, 7)])
+def test_block_size_table(n, want):
+    from bf16_huffman_infer_amd.utils import get_block_size_n
+    assert planes.get_block_size_n(n) == want
+    assert get_block_size_n(torch.empty(1, n)) == (want,)
+
+
+@pytest.mark.parametrize("n", [128, 256, 100, 4097])
+def test_block_size_rejects(n):
+    from bf16_huffman_infer_amd.utils import get_block_size_n
+    with pytest.raises(RuntimeError):
+        planes.get_block_size_n(n)
+    with pytest.raises(RuntimeError):
+        get_block_size_n(torch.empty(1, n))
+
+
+# ----------------------------------------------------------------------------- reference tables
+def test_ans_tables_worked_example():
+    sample = [1, 2, 3, 3, 2, 12, 13, 11, 1, 8, 1, 7, 1, 6, 1, 1]
+    freq, cum, lut = ref_tables.ans_tables(np.bincount(sample, minlength=256))
+    assert {s: int(f) for s, f in enumerate(freq) if f} == {1: 96, 2: 32, 3: 32, 6: 16, 7: 16, 8: 16, 11: 16,
+                                                            12: 16, 13: 16}
+    assert {s: int(cum[s]) for s in range(256) if freq[s]} == {1: 0, 2: 96, 3: 128, 6: 160, 7: 176, 8: 192,
+                                                               11: 208, 12: 224, 13: 240}
+    words, n = ref_layout._ans_words(np.array([[1]], dtype=np.uint8), freq, cum)
+    assert n[0] == 1 and words[0, 0] == 576            # 256/96 -> q=2, r=64 -> (2<<8)+64
+    e = int(lut.view(np.uint32)[576 & 255])
+    assert (e >> 24, (e >> 12) & 0xFFF, e & 0xFFF) == (1, 96, 64)
+    assert 96 * (576 >> 8) + 64 == 256
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_ans_tables_invariants_and_product_agreement(seed):
+    from bf16_huffman_infer_amd.ans import RANSEncoder
+    rng = np.random.default_rng(seed)
+    counts = np.zeros(256, dtype=np.int64)
+    syms = rng.choice(256, size=40, replace=False)
+    counts[syms] = (rng.pareto(0.7, size=40) * 50 + 1).astype(np.int64)
+    freq, cum, lut = ref_tables.ans_tables(counts)
+    assert freq.sum() == 256 and ((freq > 0) == (counts > 0)).all()
+    assert np.array_equal(cum, np.cumsum(freq) - freq)
+    u = lut.view(np.uint32)
+    for slot in range(256):
+        s, f, r = int(u[slot] >> 24), int((u[slot] >> 12) & 0xFFF), int(u[slot] & 0xFFF)
+        assert f == freq[s] and slot == cum[s] + r
+    codec = RANSEncoder(counts.tolist(), precision=8)
+    assert codec.freq == freq.tolist() and codec.cum == cum.tolist()
+    packed = [(s << 24) | (f << 12) | r for s, f, r in codec.decode_lut]
+    assert packed == u.tolist()
+
+
+@pytest.mark.parametrize("maker", [gaussian_weight, student_t_weight])
+def test_cascade_tables_decode_every_code(maker):
+    _, exp = planes.split_bf16(bits_of(maker(256, 1024, seed=4)))
+    counts = np.bincount(exp.reshape(-1), minlength=256)
+    luts, lens, codes = ref_tables.build_cascade_luts(counts)
+    kraft = sum(2.0 ** -l for _, l in codes.values())
+    assert abs(kraft - 1.0) < 1e-12 and max(l for _, l in codes.values()) <= 32
+    for s, (code, ln) in codes.items():
+        for junk in (0, 0xFFFFFFFF, 0x5A5A5A5A):
+            window = (code | (junk << ln)) & 0xFFFFFFFF
+            assert ref_tables.decode_code(luts, lens, window) == (s, ln)
+    p = counts[counts > 0] / counts.sum()
+    avg = sum(counts[s] * l for s, (_, l) in codes.items()) / counts.sum()
+    assert -(p * np.log2(p)).sum() <= avg < -(p * np.log2(p)).sum() + 1
+
+
+def test_reference_layout_index_facts():
+    idx = np.arange(256, dtype=np.uint8)[None, :]
+    so = ref_layout.stream_order(idx)
+    assert so[0, 0].tolist() == [0, 1, 128, 129] and so[0, 33].tolist() == [66, 67, 194, 195]
+    assert np.array_equal(ref_layout.stream_order_inverse(so), idx)
+    pr = ref_layout.permute_rem(np.arange(128, dtype=np.uint8)[None, :])
+    assert pr[0, :4].tolist() == [0, 1, 64, 65]
+    assert np.array_equal(ref_layout.permute_rem_inverse(pr), np.arange(128, dtype=np.uint8)[None, :])
+
+
+@pytest.mark.parametrize("maker,M,K,split_k", [(gaussian_weight, 128, 512, 1), (student_t_weight, 256, 1024, 2)])
+def test_reference_layout_round_trip(maker, M, K, split_k):
+    bits = bits_of(maker(M, K, seed=6))
+    _, exp = planes.split_bf16(bits)
+    counts = np.bincount(exp.reshape(-1), minlength=256)
+    luts, lens, codes = ref_tables.build_cascade_luts(counts)
+    enc = ref_layout.encode(bits, split_k, "huffman", codes)
+    assert enc["rem"].shape == (split_k, M, K // split_k) and enc["offsets"].shape == (split_k, M)
+    assert np.array_equal(ref_layout.decode_huffman(enc["rem"], enc["exp"], enc["offsets"], luts, lens), bits)
+    freq, cum, lut = ref_tables.ans_tables(counts)
+    enc = ref_layout.encode(bits, split_k, "ans", (freq, cum))
+    assert np.array_equal(ref_layout.decode_ans(enc["rem"], enc["exp"], enc["offsets"], lut), bits)
+
+
+def test_reference_cascade_hole_is_real():
+    """The reference reserves 255 as the miss marker, so exponent 255 (inf/NaN) cannot be
+    told from a miss; recorded here so nobody trusts the cascade on such tensors."""
+    counts = np.zeros(256, dtype=np.int64)
+    counts[[120, 121, 255]] = [1000, 900, 50]
+    luts, lens, codes = ref_tables.build_cascade_luts(counts)
+    code, ln = codes[255]
+    with pytest.raises(AssertionError):
+        assert ref_tables.decode_code(luts, lens, code) == (255, ln)
+
+
+# ----------------------------------------------------------------------------- wave64 format
+def _codec(bits):
+    from bf16_huffman_infer_amd.huffman import LUTHuffmanEncoder
+    codec = LUTHuffmanEncoder()
+    codec.build_lut(pair_counts(bits))
+    wave64.check_tables(codec.dec_table, codec.enc_table)
+    return codec
+
+
+@pytest.mark.parametrize("maker,M,K,split_k", [
+    (gaussian_weight, 128, 384, 1), (gaussian_weight, 256, 512, 2), (student_t_weight, 128, 1024, 1),
+    (random_bits_weight, 128, 384, 1), (special_values_weight, 128, 640, 1),
+    (lambda M, K, seed: torch.zeros(M, K, dtype=torch.bfloat16), 128, 128, 1),
+    (gaussian_weight, 1024, 2048, 1),
+])
+def test_wave64_round_trip(maker, M, K, split_k):
+    bits = bits_of(maker(M, K, seed=9))
+    codec = _codec(bits)
+    enc = wave64.encode(bits, split_k, codec.enc_table)
+    assert enc["rem"].shape == (split_k, M, K // split_k) and enc["offsets"].shape == (split_k, M)
+    assert len(enc["exp"]) % wave64.ALIGN_WORDS == 0
+    assert np.array_equal(wave64.decode(enc["rem"], enc["exp"], enc["offsets"], codec.dec_table), bits)
+
+
+def test_wave64_and_reference_layout_agree():
+    bits = bits_of(gaussian_weight(128, 768, seed=12))
+    codec = _codec(bits)
+    a = wave64.encode(bits, 1, codec.enc_table)
+    _, exp = planes.split_bf16(bits)
+    luts, lens, codes = ref_tables.build_cascade_luts(np.bincount(exp.reshape(-1), minlength=256))
+    b = ref_layout.encode(bits, 1, "huffman", codes)
+    da = wave64.decode(a["rem"], a["exp"], a["offsets"], codec.dec_table)
+    db = ref_layout.decode_huffman(b["rem"], b["exp"], b["offsets"], luts, lens)
+    assert np.array_equal(da, db) and np.array_equal(da, bits)
+    # the shared-stream layout has no per-row padding: it must not be larger
+    assert a["exp"].nbytes - 4 * wave64.TAIL_PAD_WORDS < b["exp"].nbytes
+
+
+def test_wave64_escape_list_and_cursor_edges():
+    """Hand-made code: three coded pairs and ESC; rows alternate so that every lane meets
+    escapes, 1-bit codes and 12-bit codes, and cursors cross words at different steps."""
+    enc = np.zeros(wave64.ESC_INDEX + 1, dtype=np.uint32)
+    dec = np.zeros(1 << wave64.TABLE_BITS, dtype=np.uint32)
+    table = {0x7878: (0b0, 1), 0x7979: (0b01, 2), 0x7A7A: (0b111111111011, 12), wave64.ESC_INDEX: (0b011111111011, 12)}
+    for p, (code, ln) in table.items():
+        enc[p] = code | (ln << 16)
+    # complete the code with filler pairs so that every 12-bit index resolves
+    filler = 0x0101
+    used = np.zeros(1 << 12, dtype=bool)
+    for p, (code, ln) in table.items():
+        idx = code + (np.arange(1 << (12 - ln)) << ln)
+        used[idx] = True
+    # every unused index becomes its own 12-bit code of a filler pair
+    for idx in np.nonzero(~used)[0]:
+        enc[filler] = int(idx) | (12 << 16)
+        table[filler] = (int(idx), 12)
+        filler += 1
+    for p, (code, ln) in table.items():
+        idx = code + (np.arange(1 << (12 - ln)) << ln)
+        dec[idx] = (ln | wave64.ESC_FLAG) if p == wave64.ESC_INDEX else (ln | ((p & 0xFF) << 7) | ((p >> 8) << 23))
+    wave64.check_tables(dec, enc)
+    rng = np.random.default_rng(0)
+    M, K = 128, 1536
+    choices = np.array([0x7878, 0x7979, 0x7A7A, 0x1234, 0xFFFE], dtype=np.uint16)   # last two are escaped
+    pr = choices[rng.choice(5, size=(M, K // 2), p=[0.55, 0.2, 0.1, 0.1, 0.05])]
+    exp = np.stack([pr & 0xFF, pr >> 8], axis=-1).reshape(M, K).astype(np.uint16)
+    bits = ((exp << 7) | rng.integers(0, 128, size=(M, K)).astype(np.uint16)
+            | (rng.integers(0, 2, size=(M, K)).astype(np.uint16) << 15)).astype(np.uint16)
+    out = wave64.encode(bits, 1, enc)
+    assert np.array_equal(wave64.decode(out["rem"], out["exp"], out["offsets"], dec), bits)
+
+
+def test_chunk_rule_matches_library():
+    from bf16_huffman_infer_amd import _lib
+    lib = _lib.load()
+    for M, Ks, sk in [(4096, 4096, 1), (4608, 3584, 1), (3584, 3584, 1), (18944, 3584, 1), (3584, 4736, 4),
+                      (12288, 4096, 1), (4096, 4096, 3), (128, 384, 1), (151936, 4096, 1), (1024, 4096, 1)]:
+        assert lib.bhi_chunks_per_group(M, Ks, sk) == wave64.chunks_per_group(M, Ks, sk)
+    c = _lib.constants()
+    assert (c["lanes"], c["group_rows"], c["step_cols"], c["table_bits"], c["window_words"], c["header_bits"],
+            c["align_words"], c["tail_pad_words"], c["target_tasks"]) == (
+        wave64.LANES, wave64.GROUP_ROWS, wave64.STEP_COLS, wave64.TABLE_BITS, wave64.WINDOW_WORDS,
+        wave64.HEADER_BITS, wave64.ALIGN_WORDS, wave64.TAIL_PAD_WORDS, wave64.TARGET_TASKS)
+
+
+# ----------------------------------------------------------------------------- pair code builder
+def test_package_merge_is_optimal_on_small_alphabets():
+    """Brute force over all length assignments with Kraft sum <= 1."""
+    from itertools import product
+    from bf16_huffman_infer_amd.huffman import package_merge
+    rng = np.random.default_rng(3)
+    for n, L in [(3, 2), (4, 3), (5, 3), (6, 3), (5, 4)]:
+        for _ in range(20):
+            w = [int(x) for x in rng.integers(1, 100, size=n)]
+            got = package_merge(w, L)
+            assert max(got) <= L and sum(2.0 ** -l for l in got) <= 1 + 1e-12
+            best = min(sum(a * b for a, b in zip(w, ls)) for ls in product(range(1, L + 1), repeat=n)
+                       if sum(2.0 ** -l for l in ls) <= 1 + 1e-12)
+            assert sum(a * b for a, b in zip(w, got)) == best
+
+
+def test_pair_code_beats_entropy_bound_plus_margin():
+    bits = bits_of(gaussian_weight(1024, 1024, seed=21))
+    counts = pair_counts(bits)
+    codec = _codec(bits)
+    p = counts[counts > 0] / counts.sum()
+    h_pair = -(p * np.log2(p)).sum()
+    avg = codec.expected_bits / counts.sum()
+    assert h_pair <= avg < h_pair + 0.2
+    assert (codec.enc_table >> 16).max() <= 12
+
+
+def test_c_abi_exports_every_declared_symbol():
+    import ctypes
+    import os
+    import re
+    from bf16_huffman_infer_amd import _lib
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "bhi.h")).read()
+    declared = set(re.findall(r"\b(bhi_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
