@@ -29,7 +29,7 @@ constexpr int kMaxBatch = 8;
 constexpr int kAnsPrecision = 8;
 constexpr int kAlignWords = 4;
 constexpr int kTailPadWords = 2048;
-constexpr int kTargetTasks = 4096;
+constexpr int kTargetTasks = 6144;      // wavefronts kept resident: 256 CUs x 4 SIMDs x 6
 constexpr int kMinChunkSteps = 4;
 constexpr int kMaxChunks = 4;
 constexpr int kMaxTaskSteps = 128;
@@ -39,7 +39,7 @@ constexpr int kBlockThreads = kWavesPerBlock * kLanes;
 __host__ __device__ inline int chunks_per_group(int M, int Ks, int split_k) {
     int steps = Ks / kStepCols;
     int nc = 1;
-    while (nc < kMaxChunks && (long long)(M / kGroupRows) * split_k * nc < kTargetTasks &&
+    while (nc < kMaxChunks && (long long)(M / kGroupRows) * split_k * nc * 2 <= kTargetTasks &&
            steps / (nc * 2) >= kMinChunkSteps)
         nc *= 2;
     return nc;
@@ -82,22 +82,21 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
     return s;
 }
 
-// A task is processed in segments of kSegSteps steps: load phase (every global load of
-// the segment issued back to back, unconditionally, with clamped indices), then compute
-// phase (no global loads).  VMEM loads complete in issue order, so a load placed inside
-// the compute phase would make its wait drain the whole queue; latency is hidden by the
-// other wavefronts of the SIMD being in a different phase.
+// A task is processed in segments of kSegSteps steps; the global loads of a segment
+// (all unconditional, with clamped indices) are issued one segment ahead of their use.
+// VMEM loads complete in issue order, so a load issued on demand inside a segment would
+// make its wait drain the whole queue.
 //
-// Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each).
-// Row r lives in slot r % kRingRows; slots 0 and 1 are mirrored behind the last slot so
-// that the three rows of a lane's window are always at +0, +256 and +512 bytes.  Lanes
-// sit at different rows, yet row r of lane l is always in bank l % 32: window reads are
-// conflict free.  The ring is topped up when some lane's window is about to leave the
-// staged rows (a cheap per-step test); a lane that is more than a ring ahead of the
-// slowest lane reads its window from global memory instead.
-constexpr int kSegSteps = 8;
+// Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each,
+// the ring is aligned to its 4 KB size so that a slot address is an AND and an OR).
+// Row r lives in slot r % kRingRows.  Lanes sit at different rows, yet row r of lane l
+// is always in bank l % 32: window reads are conflict free.  Every segment prefetches the next kSegRows rows and commits them to
+// the ring once the previous segment is decoded; a lane whose window is not staged (a
+// cheap per-step test) reads it from global memory instead.
+constexpr int kSegSteps = 4;
 constexpr int kRingRows = 16;
-constexpr int kRingSlots = kRingRows + 2;
+constexpr int kSegRows = 6;          // rows prefetched per segment = the most a lane can consume in one
+constexpr int kRingSlots = kRingRows;
 constexpr int kRingWords = kRingSlots * kLanes;
 
 // LDS pointers are kept in their own address space: a pointer that may be LDS or global
@@ -135,26 +134,61 @@ struct HuffCursor {
         eptr = 0;
     }
 
-    // Stage rows up to kRingRows past the slowest lane.  Global loads + LDS stores.
-    __device__ __forceinline__ void top_up() {
+    // LDS address of this lane's word of row (p >> 5) + k: the ring base has its bits
+    // 8..11 clear, the row index lands there.
+    __device__ __forceinline__ const lds_u32* slot_of(uint32_t p, int k) const {
+        const uint32_t off = ((p << 3) + 256u * k) & ((kRingRows - 1) * 256u);
+        return (const lds_u32*)(off | (uint32_t)(uintptr_t)ring);
+    }
+
+    // Stage the first rows of the block (once per task; the loads are waited for here).
+    __device__ __forceinline__ void prime() {
+        const uint32_t hi = nrows < (uint32_t)kRingRows ? nrows : (uint32_t)kRingRows;
+        uint32_t v[kRingRows];
+#pragma unroll
+        for (int j = 0; j < kRingRows; ++j) {
+            const uint32_t r = (uint32_t)j < nrows ? (uint32_t)j : nrows - 1;
+            v[j] = bp[(size_t)r * kLanes];
+        }
+#pragma unroll
+        for (int j = 0; j < kRingRows; ++j) {
+            ring[j * kLanes] = v[j];
+        }
+        rhi = hi;
+        set_lim();
+    }
+
+    // windows read rows m..m+2; once the whole block is staged nothing can be missing
+    __device__ __forceinline__ void set_lim() {
+        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi >= 2 ? (rhi - 2) << 5 : 0u);
+    }
+
+    // Load phase: the next kSegRows rows after the staged ones, unconditionally (clamped).
+    __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) const {
+#pragma unroll
+        for (int j = 0; j < kSegRows; ++j) {
+            uint32_t r = rhi + j;
+            r = r < nrows ? r : nrows - 1;
+            v[j] = bp[(size_t)r * kLanes];
+        }
+    }
+
+    // Start of the compute phase: move the prefetched rows into the ring as far as the
+    // slowest lane allows (row r may replace row r - kRingRows once no window needs it).
+    __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
         const uint32_t mmin = uniform(wave_min(pos) >> 5);
         uint32_t hi = mmin + kRingRows;
         hi = hi < nrows ? hi : nrows;
-        uint32_t v[kRingRows];
+        hi = hi < rhi + kSegRows ? hi : rhi + kSegRows;
 #pragma unroll
-        for (int j = 0; j < kRingRows; ++j)
-            if (rhi + j < hi) v[j] = bp[(size_t)(rhi + j) * kLanes];
-#pragma unroll
-        for (int j = 0; j < kRingRows; ++j) {
+        for (int j = 0; j < kSegRows; ++j) {
             if (rhi + j < hi) {
                 const uint32_t slot = (rhi + j) & (kRingRows - 1);
                 ring[slot * kLanes] = v[j];
-                if (slot < 2) ring[(kRingRows + slot) * kLanes] = v[j];
             }
         }
         rhi = hi > rhi ? hi : rhi;
-        // windows read rows m..m+2; once the whole block is staged nothing can be missing
-        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi >= 2 ? (rhi - 2) << 5 : 0u);
+        set_lim();
     }
 
     // Decode the four pairs of one step; e[q] are raw table entries.
@@ -162,13 +196,11 @@ struct HuffCursor {
     __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
         uint32_t lo, hi, nx;
         if (__builtin_expect(ballot(pos >= lim) != 0, 0)) {
-            top_up();
             fetch_slow(lo, hi, nx);
         } else {
-            const lds_u32* w = ring + ((pos >> 5) & (kRingRows - 1)) * kLanes;
-            lo = w[0];
-            hi = w[kLanes];
-            nx = w[2 * kLanes];
+            lo = *slot_of(pos, 0);
+            hi = *slot_of(pos, 1);
+            nx = *slot_of(pos, 2);
         }
         const char* tb = (const char*)table;
         const uint32_t c = pos & 31u;
@@ -198,14 +230,13 @@ struct HuffCursor {
         }
     }
 
-    // After a top-up: lanes whose window is staged read the ring, the others (more than
-    // a ring ahead of the slowest lane) read global memory.
+    // Some lane's window is not staged (it ran more than a ring ahead of the slowest lane,
+    // or further than one segment's prefetch): those lanes read global memory.
     __device__ __forceinline__ void fetch_slow(uint32_t& lo, uint32_t& hi, uint32_t& nx) {
         const uint32_t m = pos >> 5;
         const bool staged = pos < lim;
         // clamp so that both reads are always in range, then pick per lane
-        const lds_u32* w = ring + (m & (kRingRows - 1)) * kLanes;
-        const uint32_t l0 = w[0], l1 = w[kLanes], l2 = w[2 * kLanes];
+        const uint32_t l0 = *slot_of(pos, 0), l1 = *slot_of(pos, 1), l2 = *slot_of(pos, 2);
         const uint32_t* g = bp + (size_t)(staged ? 0u : m) * kLanes;
         const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
         lo = staged ? l0 : g0;

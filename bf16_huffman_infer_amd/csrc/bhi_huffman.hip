@@ -25,35 +25,56 @@ struct Shape {
     uint32_t total_words;
 };
 
-// Runs one task segment by segment.  A policy supplies the operands that travel with
-// the exponent stream: `Slot` holds what is loaded for a whole segment in the load
-// phase (`load(slot, t)`, t clamped by the policy); `take(...)` hands out what the
-// policy pipelines on its own inside the compute phase; `use(...)` receives the
-// lane's four rebuilt BF16 pairs (columns 0..7 of its row in step t).
+// Runs one task as a two-stage software pipeline over segments of kSegSteps steps: while
+// segment s is decoded, the loads of segment s+1 (operand slots and the next exponent
+// rows) are in flight.  A policy supplies the operands that travel with the exponent
+// stream: `Slot` holds what is loaded per step (`load(slot, t)`, t clamped by the
+// policy); `take(...)` hands out what the policy pipelines on its own inside the
+// compute phase; `use(...)` receives the lane's four rebuilt BF16 pairs (columns 0..7
+// of its row in step t).  Every global load is unconditional, so the compiler can
+// count outstanding loads and wait for exactly the ones a step needs.
+template <class Policy>
+__device__ __forceinline__ void load_segment(const Policy& pol, typename Policy::Slot (&slot)[kSegSteps], int t0) {
+#pragma unroll
+    for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], t0 + i);
+}
+
+template <bool HAS_ESC, class Policy>
+__device__ __forceinline__ void decode_segment(HuffCursor& cur, const uint32_t* lut, Policy& pol,
+                                               const typename Policy::Slot (&slot)[kSegSteps], int t0, int ns) {
+#pragma unroll
+    for (int i = 0; i < kSegSteps; ++i) {
+        if (t0 + i < ns) {
+            const typename Policy::Piped piped = pol.take(slot[i], i, t0 + i);
+            uint32_t e[4];
+            cur.template step<HAS_ESC>(lut, e);
+            uint32_t w[4];
+            const uint2 r = slot[i].rem;
+            w[0] = rebuild_pair(e[0], rem_lo_pair(r.x));
+            w[1] = rebuild_pair(e[1], rem_hi_pair(r.x));
+            w[2] = rebuild_pair(e[2], rem_lo_pair(r.y));
+            w[3] = rebuild_pair(e[3], rem_hi_pair(r.y));
+            pol.use(piped, t0 + i, w);
+        }
+    }
+}
+
 template <bool HAS_ESC, class Policy>
 __device__ __forceinline__ void run_task(HuffCursor& cur, const uint32_t* lut, Policy& pol, int ns) {
+    typename Policy::Slot sa[kSegSteps], sb[kSegSteps];
+    uint32_t ra[kSegRows], rb[kSegRows];
     pol.prime();
-    for (int seg = 0; seg < ns; seg += kSegSteps) {
-        // ---- load phase: nothing but global loads, all unconditional
-        typename Policy::Slot slot[kSegSteps];
-#pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], seg + i);
-        // ---- compute phase
-#pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) {
-            if (seg + i < ns) {
-                const typename Policy::Piped piped = pol.take(slot[i], i, seg + i);
-                uint32_t e[4];
-                cur.template step<HAS_ESC>(lut, e);
-                uint32_t w[4];
-                const uint2 r = slot[i].rem;
-                w[0] = rebuild_pair(e[0], rem_lo_pair(r.x));
-                w[1] = rebuild_pair(e[1], rem_hi_pair(r.x));
-                w[2] = rebuild_pair(e[2], rem_lo_pair(r.y));
-                w[3] = rebuild_pair(e[3], rem_hi_pair(r.y));
-                pol.use(piped, seg + i, w);
-            }
-        }
+    load_segment(pol, sa, 0);
+    cur.prime();
+    for (int seg = 0; seg < ns; seg += 2 * kSegSteps) {
+        cur.prefetch(rb);
+        load_segment(pol, sb, seg + kSegSteps);
+        decode_segment<HAS_ESC>(cur, lut, pol, sa, seg, ns);
+        cur.commit(rb);
+        cur.prefetch(ra);
+        load_segment(pol, sa, seg + 2 * kSegSteps);
+        decode_segment<HAS_ESC>(cur, lut, pol, sb, seg + kSegSteps, ns);
+        cur.commit(ra);
     }
 }
 
@@ -177,8 +198,8 @@ __global__ __launch_bounds__(NW * kLanes)
 void huffman_decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
                            uint16_t* __restrict__ Y, const uint32_t* __restrict__ offsets,
                            const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
+    __shared__ __align__(4096) uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[kTableEntries];
-    __shared__ uint32_t rings[NW][kRingWords];
     load_table(lut, table);
     __syncthreads();
 
@@ -208,17 +229,17 @@ void huffman_decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __
 // P = min(split_k*nc, NW) wavefronts of the same block (a wavefront loops when there
 // are more tasks than that), so the sum over splits and chunks never leaves the block.
 // register budget: at least this many wavefronts per SIMD must stay resident
-constexpr int min_waves(int bs) { return bs <= 1 ? 6 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
+constexpr int min_waves(int bs) { return bs <= 2 ? 5 : (bs <= 4 ? 4 : 3); }
 
 template <int BS, int NW>
-__global__ __launch_bounds__(NW * kLanes)
+__global__ __launch_bounds__(NW * kLanes, min_waves(BS))
 void gemv_huffman_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
                          const uint16_t* __restrict__ X, uint16_t* __restrict__ Y,
                          const uint32_t* __restrict__ offsets, const uint32_t* __restrict__ table,
                          const uint8_t* __restrict__ header, Shape s, int P, int groups_per_block) {
     // The partial sums reuse the rings once every task of the block is done.
+    __shared__ __align__(4096) uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[kTableEntries];
-    __shared__ uint32_t rings[NW][kRingWords];
     load_table(lut, table);
     __syncthreads();
 

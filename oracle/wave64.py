@@ -55,7 +55,7 @@ WINDOW_WORDS = 3           # words of its bitstring a lane looks at per step
 HEADER_BITS = 2            # dummy bits in front of every lane's codes
 TABLE_BITS = 12
 ESC_FLAG = 1 << 15
-TARGET_TASKS = 4096
+TARGET_TASKS = 6144        # wavefronts one MI355X keeps resident: 256 CUs x 4 SIMDs x 6
 MIN_CHUNK_STEPS = 4
 MAX_CHUNKS = 4
 ALIGN_WORDS = 4
@@ -67,7 +67,7 @@ def chunks_per_group(M: int, Ks: int, split_k: int) -> int:
     """How many independent streams a (split, row group) is cut into."""
     steps = Ks // STEP_COLS
     nc = 1
-    while (nc < MAX_CHUNKS and (M // GROUP_ROWS) * split_k * nc < TARGET_TASKS
+    while (nc < MAX_CHUNKS and (M // GROUP_ROWS) * split_k * nc * 2 <= TARGET_TASKS
            and steps // (nc * 2) >= MIN_CHUNK_STEPS):
         nc *= 2
     return nc
