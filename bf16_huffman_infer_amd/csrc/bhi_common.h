@@ -93,9 +93,10 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
 // is always in bank l % 32: window reads are conflict free.  Every segment prefetches the next kSegRows rows and commits them to
 // the ring once the previous segment is decoded; a lane whose window is not staged (a
 // cheap per-step test) reads it from global memory instead.
-constexpr int kSegSteps = 4;
+constexpr bool kPipelined = false;
+constexpr int kSegSteps = 8;
 constexpr int kRingRows = 16;
-constexpr int kSegRows = 6;          // rows prefetched per segment = the most a lane can consume in one
+constexpr int kSegRows = 8;          // rows prefetched per segment = the most a lane can consume in one
 constexpr int kRingSlots = kRingRows;
 constexpr int kRingWords = kRingSlots * kLanes;
 

@@ -61,20 +61,32 @@ __device__ __forceinline__ void decode_segment(HuffCursor& cur, const uint32_t* 
 
 template <bool HAS_ESC, class Policy>
 __device__ __forceinline__ void run_task(HuffCursor& cur, const uint32_t* lut, Policy& pol, int ns) {
-    typename Policy::Slot sa[kSegSteps], sb[kSegSteps];
-    uint32_t ra[kSegRows], rb[kSegRows];
     pol.prime();
-    load_segment(pol, sa, 0);
-    cur.prime();
-    for (int seg = 0; seg < ns; seg += 2 * kSegSteps) {
-        cur.prefetch(rb);
-        load_segment(pol, sb, seg + kSegSteps);
-        decode_segment<HAS_ESC>(cur, lut, pol, sa, seg, ns);
-        cur.commit(rb);
-        cur.prefetch(ra);
-        load_segment(pol, sa, seg + 2 * kSegSteps);
-        decode_segment<HAS_ESC>(cur, lut, pol, sb, seg + kSegSteps, ns);
-        cur.commit(ra);
+    if (kPipelined) {
+        typename Policy::Slot sa[kSegSteps], sb[kSegSteps];
+        uint32_t ra[kSegRows], rb[kSegRows];
+        load_segment(pol, sa, 0);
+        cur.prime();
+        for (int seg = 0; seg < ns; seg += 2 * kSegSteps) {
+            cur.prefetch(rb);
+            load_segment(pol, sb, seg + kSegSteps);
+            decode_segment<HAS_ESC>(cur, lut, pol, sa, seg, ns);
+            cur.commit(rb);
+            cur.prefetch(ra);
+            load_segment(pol, sa, seg + 2 * kSegSteps);
+            decode_segment<HAS_ESC>(cur, lut, pol, sb, seg + kSegSteps, ns);
+            cur.commit(ra);
+        }
+    } else {
+        cur.prime();
+        for (int seg = 0; seg < ns; seg += kSegSteps) {
+            typename Policy::Slot slot[kSegSteps];
+            uint32_t rows[kSegRows];
+            if (seg) cur.prefetch(rows);
+            load_segment(pol, slot, seg);
+            if (seg) cur.commit(rows);
+            decode_segment<HAS_ESC>(cur, lut, pol, slot, seg, ns);
+        }
     }
 }
 
@@ -229,7 +241,7 @@ void huffman_decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __
 // P = min(split_k*nc, NW) wavefronts of the same block (a wavefront loops when there
 // are more tasks than that), so the sum over splits and chunks never leaves the block.
 // register budget: at least this many wavefronts per SIMD must stay resident
-constexpr int min_waves(int bs) { return bs <= 2 ? 5 : (bs <= 4 ? 4 : 3); }
+constexpr int min_waves(int bs) { return bs <= 1 ? 6 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
 
 template <int BS, int NW>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
@@ -427,7 +439,7 @@ static void launch_gemv(const void* A_rem, const void* A_exp, const void* X, voi
     const int G = s.M / kGroupRows;
     // small blocks spread more evenly over the 256 CUs; 8 wavefronts only when one row
     // group needs more than 4 of them
-    if (per_group <= 4) {
+    if (false) {
         constexpr int NW = 4;
         const int P = per_group, gpb = NW / P;
         hipLaunchKernelGGL((gemv_huffman_kernel<BS, NW>), dim3((unsigned)((G + gpb - 1) / gpb)), dim3(NW * kLanes), 0, stream,
