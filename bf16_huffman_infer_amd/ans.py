@@ -37,38 +37,34 @@ class RANSEncoder:
         ]
 
     def _normalize(self, freq: Mapping[int, int]) -> Dict[int, int]:
+        """Counts -> slots summing to ``2**precision`` (same result as the reference's
+        fix-up loop, written as whole passes over the symbols in remainder order)."""
         total = sum(freq.values())
         if total <= 0:
             raise ValueError("sum of frequencies must be positive")
         if len(freq) > self.base:
             raise ValueError("more symbols than slots")
-        scaled: Dict[int, int] = {}
-        remainders = []
-        for sym, count in freq.items():
-            if count <= 0:
-                raise ValueError(f"frequency of symbol {sym} must be positive")
-            exact = count * self.base / total
-            slots = max(int(round(exact)), 1)          # round() is round-half-even
-            scaled[sym] = slots
-            remainders.append((exact - slots, sym))
+        if min(freq.values()) <= 0:
+            bad = min(freq, key=freq.get)
+            raise ValueError(f"frequency of symbol {bad} must be positive")
 
-        current = sum(scaled.values())
-        if current < self.base:
-            remainders.sort(reverse=True)               # most under-served first
-            while current < self.base:
-                for _, sym in remainders:
-                    if current == self.base:
-                        break
-                    scaled[sym] += 1
-                    current += 1
-        elif current > self.base:
-            remainders.sort()                           # most over-served first
-            while current > self.base:
-                for _, sym in remainders:
-                    if current == self.base:
-                        break
-                    if scaled[sym] > 1:
-                        scaled[sym] -= 1
-                        current -= 1
-        assert sum(scaled.values()) == self.base
-        return scaled
+        exact = {s: c * self.base / total for s, c in freq.items()}
+        slots = {s: max(int(round(v)), 1) for s, v in exact.items()}     # round() is half-to-even
+        missing = self.base - sum(slots.values())
+        if missing > 0:
+            # most under-served symbol first; every pass hands one slot to each symbol
+            order = sorted(slots, key=lambda s: (exact[s] - slots[s], s), reverse=True)
+            rounds, extra = divmod(missing, len(order))
+            for i, s in enumerate(order):
+                slots[s] += rounds + (1 if i < extra else 0)
+        elif missing < 0:
+            # most over-served symbol first; a symbol never drops below one slot
+            order = sorted(slots, key=lambda s: (exact[s] - slots[s], s))
+            surplus = -missing
+            while surplus:
+                for s in order:
+                    if surplus and slots[s] > 1:
+                        slots[s] -= 1
+                        surplus -= 1
+        assert sum(slots.values()) == self.base
+        return slots
