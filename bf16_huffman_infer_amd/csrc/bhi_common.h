@@ -113,33 +113,30 @@ __device__ __forceinline__ uint32_t wave_min(uint32_t v) {
     return v;
 }
 
-// Per-lane Huffman bit cursor over the lane's rows of the task block.
-struct HuffCursor {
-    uint32_t pos;            // bit position - 2 (the window is kept shifted left by two)
+// A lane's view of its task block: a bit position in its own column of rows, and the
+// wavefront's LDS ring of staged rows.  The codec cursors below build on it.
+struct RowRing {
+    uint32_t pos;            // bit position of the lane's window (codec specific bias)
     uint32_t rhi;            // wave-uniform: rows [0, rhi) have been staged
     uint32_t lim;            // wave-uniform: windows starting below this bit are fully staged
     uint32_t nrows;          // wave-uniform: rows of the block worth staging
-    uint32_t eptr;           // wave-uniform: escape entries consumed so far
     const uint32_t* bp;      // task block, this lane's column
-    const uint32_t* ep;      // one past the task block (escape list grows down from here)
     lds_u32* ring;           // this wavefront's LDS ring, this lane's column
 
-    __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t* ring_) {
+    __device__ __forceinline__ void open_rows(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t* ring_) {
         bp = words + span.base + lane;
-        ep = words + span.end;
         ring = (lds_u32*)ring_ + lane;
         nrows = uniform((span.end - span.base + kLanes - 1) / kLanes);
         pos = 0;
         rhi = 0;
         lim = 0;
-        eptr = 0;
     }
 
     // LDS address of this lane's word of row (p >> 5) + k: the ring base has its bits
     // 8..11 clear, the row index lands there.
     __device__ __forceinline__ const lds_u32* slot_of(uint32_t p, int k) const {
         const uint32_t off = ((p << 3) + 256u * k) & ((kRingRows - 1) * 256u);
-        return (const lds_u32*)(off | (uint32_t)(uintptr_t)ring);
+        return (const lds_u32*)(uintptr_t)(off | (uint32_t)(uintptr_t)ring);
     }
 
     // Stage the first rows of the block (once per task; the loads are waited for here).
@@ -152,9 +149,7 @@ struct HuffCursor {
             v[j] = bp[(size_t)r * kLanes];
         }
 #pragma unroll
-        for (int j = 0; j < kRingRows; ++j) {
-            ring[j * kLanes] = v[j];
-        }
+        for (int j = 0; j < kRingRows; ++j) ring[j * kLanes] = v[j];
         rhi = hi;
         set_lim();
     }
@@ -164,7 +159,7 @@ struct HuffCursor {
         lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi >= 2 ? (rhi - 2) << 5 : 0u);
     }
 
-    // Load phase: the next kSegRows rows after the staged ones, unconditionally (clamped).
+    // The next kSegRows rows after the staged ones, unconditionally (clamped).
     __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) const {
 #pragma unroll
         for (int j = 0; j < kSegRows; ++j) {
@@ -174,8 +169,8 @@ struct HuffCursor {
         }
     }
 
-    // Start of the compute phase: move the prefetched rows into the ring as far as the
-    // slowest lane allows (row r may replace row r - kRingRows once no window needs it).
+    // Move the prefetched rows into the ring as far as the slowest lane allows (row r may
+    // replace row r - kRingRows once no window needs it).
     __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
         const uint32_t mmin = uniform(wave_min(pos) >> 5);
         uint32_t hi = mmin + kRingRows;
@@ -192,10 +187,8 @@ struct HuffCursor {
         set_lim();
     }
 
-    // Decode the four pairs of one step; e[q] are raw table entries.
-    template <bool HAS_ESC>
-    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
-        uint32_t lo, hi, nx;
+    // The lane's window: rows m, m+1, m+2 with m = pos >> 5.
+    __device__ __forceinline__ void window(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
         if (__builtin_expect(ballot(pos >= lim) != 0, 0)) {
             fetch_slow(lo, hi, nx);
         } else {
@@ -203,6 +196,42 @@ struct HuffCursor {
             hi = *slot_of(pos, 1);
             nx = *slot_of(pos, 2);
         }
+    }
+
+    // Some lane's window is not staged (it ran more than a ring ahead of the slowest lane,
+    // or further than one segment's prefetch): those lanes read global memory.
+    __device__ __forceinline__ void fetch_slow(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
+        const uint32_t m = pos >> 5;
+        const bool staged = pos < lim;
+        // both reads are always in range (the stream ends in a zero pad), then pick per lane
+        const uint32_t l0 = *slot_of(pos, 0), l1 = *slot_of(pos, 1), l2 = *slot_of(pos, 2);
+        const uint32_t* g = bp + (size_t)(staged ? 0u : m) * kLanes;
+        const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
+        lo = staged ? l0 : g0;
+        hi = staged ? l1 : g1;
+        nx = staged ? l2 : g2;
+    }
+};
+
+// Per-lane Huffman bit cursor.  pos = bit position - 2: the window is kept shifted left
+// by two so that `window & 0x3FFC` is the byte address of the table entry.
+struct HuffCursor : RowRing {
+    uint32_t eptr;           // wave-uniform: escape entries consumed so far
+    const uint32_t* ep;      // one past the task block (escape list grows down from here)
+
+    __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t* ring_) {
+        open_rows(words, span, lane, ring_);
+        ep = words + span.end;
+        eptr = 0;
+    }
+
+    __device__ __forceinline__ void start() {}
+
+    // Decode the four pairs of one step; e[q] are raw table entries.
+    template <bool HAS_ESC>
+    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
+        uint32_t lo, hi, nx;
+        window(lo, hi, nx);
         const char* tb = (const char*)table;
         const uint32_t c = pos & 31u;
         const uint32_t wlo = __builtin_amdgcn_alignbit(hi, lo, c);
@@ -231,20 +260,6 @@ struct HuffCursor {
         }
     }
 
-    // Some lane's window is not staged (it ran more than a ring ahead of the slowest lane,
-    // or further than one segment's prefetch): those lanes read global memory.
-    __device__ __forceinline__ void fetch_slow(uint32_t& lo, uint32_t& hi, uint32_t& nx) {
-        const uint32_t m = pos >> 5;
-        const bool staged = pos < lim;
-        // clamp so that both reads are always in range, then pick per lane
-        const uint32_t l0 = *slot_of(pos, 0), l1 = *slot_of(pos, 1), l2 = *slot_of(pos, 2);
-        const uint32_t* g = bp + (size_t)(staged ? 0u : m) * kLanes;
-        const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
-        lo = staged ? l0 : g0;
-        hi = staged ? l1 : g1;
-        nx = staged ? l2 : g2;
-    }
-
     // Exponents of escaped pairs come from the escape list, in (pair, lane) order.
     __device__ __forceinline__ void escapes(uint32_t (&e)[4]) {
 #pragma unroll
@@ -257,6 +272,63 @@ struct HuffCursor {
             }
             eptr = uniform(eptr + (uint32_t)__builtin_popcountll(m));
         }
+    }
+};
+
+// Per-lane rANS cursor: one 64-bit state, precision 8, table words (sym<<24)|(freq<<12)|rem.
+// The state is looked at after every four symbols; when it has dropped below 2**32 the
+// lane's next row word is shifted in.  pos = 32 * (index of the lane's next row).
+struct AnsCursor : RowRing {
+    uint32_t xl, xh;         // the state
+
+    __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t* ring_) {
+        open_rows(words, span, lane, ring_);
+    }
+
+    // rows 0 and 1 are the initial state (call after prime())
+    __device__ __forceinline__ void start() {
+        xl = ring[0];
+        xh = ring[kLanes];
+        pos = 2 * 32;
+    }
+
+    // one symbol: returns the table word, advances the state
+    __device__ __forceinline__ uint32_t symbol(const uint32_t* __restrict__ table) {
+        const uint32_t ent = *(const uint32_t*)((const char*)table + ((xl & 0xFFu) << 2));
+        const uint32_t f = (ent >> 12) & 0xFFFu;
+        const uint32_t yl = __builtin_amdgcn_alignbit(xh, xl, 8);
+        const uint32_t yh = xh >> 8;
+        const uint64_t lowp = (uint64_t)f * yl + (ent & 0xFFFu);      // v_mad_u64_u32
+        xl = (uint32_t)lowp;
+        xh = (uint32_t)(lowp >> 32) + f * yh;                         // f * yh < 2**33 only if the state is valid: < 2**32
+        return ent;
+    }
+
+    __device__ __forceinline__ void refill(uint32_t word) {
+        const bool need = xh == 0u;
+        xh = need ? xl : xh;
+        xl = need ? word : xl;
+        pos += need ? 32u : 0u;
+    }
+
+    // two symbols -> one pair entry in the Huffman table's format (a<<7 | b<<23)
+    __device__ __forceinline__ uint32_t pair(const uint32_t* __restrict__ table) {
+        const uint32_t a = symbol(table);
+        const uint32_t b = symbol(table);
+        return ((a >> 17) & 0x7F80u) | ((b >> 1) & 0x7F800000u);
+    }
+
+    template <bool UNUSED>
+    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
+        uint32_t lo, hi, nx;
+        window(lo, hi, nx);
+        e[0] = pair(table);
+        e[1] = pair(table);
+        const bool first = xh == 0u;
+        refill(lo);
+        e[2] = pair(table);
+        e[3] = pair(table);
+        refill(first ? hi : lo);
     }
 };
 

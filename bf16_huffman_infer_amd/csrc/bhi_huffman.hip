@@ -3,328 +3,18 @@
 // Stand-ins for the reference's gemv_bf16_huffman / huffman_decode / huffman_encode
 // (bf16_huffman_infer/src/kernel.cu:419-442, 510-531, 590-610).  The reference walks
 // one row per 32-lane warp with two private bitstreams per lane and two dependent
-// byte-table reads per exponent; here one 64-lane wavefront walks four rows, one LDS
-// read resolves two exponents, and all lanes share one refill stream.
-#include "bhi_common.h"
-#include "bhi_host.h"
+// byte-table reads per exponent; here one 64-lane wavefront walks four rows and one LDS
+// read resolves two exponents.
+#include "bhi_task.h"
 
 namespace bhi {
 
-typedef short bf16x4_t __attribute__((ext_vector_type(4)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
-// Cooperative copy of the 16 KB pair table into LDS.
-__device__ __forceinline__ void load_table(uint32_t* __restrict__ lds, const uint32_t* __restrict__ g) {
-    const uint4* src = (const uint4*)g;
-    uint4* dst = (uint4*)lds;
-    for (int i = threadIdx.x; i < kTableEntries / 4; i += blockDim.x) dst[i] = src[i];
-}
-
-struct Shape {
-    int M, Ks, split_k, nc, steps;      // steps per (split, group)
-    uint32_t total_words;
+struct HuffCodec {
+    using Cursor = HuffCursor;
+    static constexpr int kTableWords = kTableEntries;
+    // escaped pairs need the slower walk; the header says whether the matrix has any
+    static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ header) { return header_has_esc(header); }
 };
-
-// Runs one task as a two-stage software pipeline over segments of kSegSteps steps: while
-// segment s is decoded, the loads of segment s+1 (operand slots and the next exponent
-// rows) are in flight.  A policy supplies the operands that travel with the exponent
-// stream: `Slot` holds what is loaded per step (`load(slot, t)`, t clamped by the
-// policy); `take(...)` hands out what the policy pipelines on its own inside the
-// compute phase; `use(...)` receives the lane's four rebuilt BF16 pairs (columns 0..7
-// of its row in step t).  Every global load is unconditional, so the compiler can
-// count outstanding loads and wait for exactly the ones a step needs.
-template <class Policy>
-__device__ __forceinline__ void load_segment(const Policy& pol, typename Policy::Slot (&slot)[kSegSteps], int t0) {
-#pragma unroll
-    for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], t0 + i);
-}
-
-template <bool HAS_ESC, class Policy>
-__device__ __forceinline__ void decode_segment(HuffCursor& cur, const uint32_t* lut, Policy& pol,
-                                               const typename Policy::Slot (&slot)[kSegSteps], int t0, int ns) {
-#pragma unroll
-    for (int i = 0; i < kSegSteps; ++i) {
-        if (t0 + i < ns) {
-            const typename Policy::Piped piped = pol.take(slot[i], i, t0 + i);
-            uint32_t e[4];
-            cur.template step<HAS_ESC>(lut, e);
-            uint32_t w[4];
-            const uint2 r = slot[i].rem;
-            w[0] = rebuild_pair(e[0], rem_lo_pair(r.x));
-            w[1] = rebuild_pair(e[1], rem_hi_pair(r.x));
-            w[2] = rebuild_pair(e[2], rem_lo_pair(r.y));
-            w[3] = rebuild_pair(e[3], rem_hi_pair(r.y));
-            pol.use(piped, t0 + i, w);
-        }
-    }
-}
-
-template <bool HAS_ESC, class Policy>
-__device__ __forceinline__ void run_task(HuffCursor& cur, const uint32_t* lut, Policy& pol, int ns) {
-    pol.prime();
-    if (kPipelined) {
-        typename Policy::Slot sa[kSegSteps], sb[kSegSteps];
-        uint32_t ra[kSegRows], rb[kSegRows];
-        load_segment(pol, sa, 0);
-        cur.prime();
-        for (int seg = 0; seg < ns; seg += 2 * kSegSteps) {
-            cur.prefetch(rb);
-            load_segment(pol, sb, seg + kSegSteps);
-            decode_segment<HAS_ESC>(cur, lut, pol, sa, seg, ns);
-            cur.commit(rb);
-            cur.prefetch(ra);
-            load_segment(pol, sa, seg + 2 * kSegSteps);
-            decode_segment<HAS_ESC>(cur, lut, pol, sb, seg + kSegSteps, ns);
-            cur.commit(ra);
-        }
-    } else {
-        cur.prime();
-        for (int seg = 0; seg < ns; seg += kSegSteps) {
-            typename Policy::Slot slot[kSegSteps];
-            uint32_t rows[kSegRows];
-            if (seg) cur.prefetch(rows);
-            load_segment(pol, slot, seg);
-            if (seg) cur.commit(rows);
-            decode_segment<HAS_ESC>(cur, lut, pol, slot, seg, ns);
-        }
-    }
-}
-
-// The format header (code_lengths buffer): [0] version, [1] table bits, [2] ESC code
-// length, [3] nonzero when the matrix contains escaped pairs.
-__device__ __forceinline__ bool header_has_esc(const uint8_t* __restrict__ header) {
-    return uniform(header[3]) != 0;
-}
-
-// decode-to-BF16: rem in, 16 bytes of weights out per lane and step
-struct StorePolicy {
-    struct Slot { uint2 rem; };
-    struct Piped {};
-    const uint2* rem0;       // this lane's 8 rem bytes of the task's first step
-    uint16_t* yp;            // this lane's 8 output columns of the task's first step
-    int last;
-
-    __device__ __forceinline__ void prime() const {}
-    __device__ __forceinline__ void load(Slot& s, int t) const {
-        t = t < last ? t : last;
-        s.rem = rem0[(size_t)t * kLanes];
-    }
-    __device__ __forceinline__ Piped take(const Slot&, int, int) const { return Piped{}; }
-    __device__ __forceinline__ void use(const Piped&, int t, const uint32_t (&w)[4]) const {
-        *(uint4*)(yp + (size_t)t * kStepCols) = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-};
-
-// Broadcast of lane q of every quad (dpp quad_perm:[q,q,q,q]).
-template <int Q>
-__device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, Q * 0x55, 0xF, 0xF, true);
-}
-
-// fused GEMV on the matrix cores: v_mfma_f32_4x4x4_16b_bf16 multiplies, in each of its
-// 16 blocks, 4 rows x 4 k (operand A: lane 4*blk + row holds the 4 k values of that row)
-// by 4 k x 4 columns (operand B: lane 4*blk + col) into D[row][col] (register `row` of lane
-// 4*blk + col).  A lane's four pairs are exactly two A operands (columns 0..3 and 4..7 of
-// its row); lane 4*b + j supplies X[batch j] for those columns.  One accumulator set
-// covers batches 0..3, a second one batches 4..7.  Lanes whose batch does not exist
-// carry finite filler and their results are never stored.
-//
-// How X reaches the B operand depends on the batch:
-//   batch 1     the four lanes of a quad own the same 8 columns; each loads one X pair
-//               in the load phase (one register per step) and the quad shares them by DPP;
-//   batch 2..4  every lane loads its batch's 8 columns in the load phase (4 registers/step);
-//   batch 5..8  two sets would need 8 registers per step: X is fetched two steps ahead
-//               inside the compute phase instead (it is cache resident).
-template <int BS>
-struct MfmaPolicy {
-    static constexpr int NSET = BS <= 4 ? 1 : 2;
-    static constexpr bool QUARTER = BS == 1;
-    static constexpr bool PIPED = BS > 4;
-    static constexpr int XAHEAD = 2;
-    struct Slot { uint2 rem; uint4 x; };         // x: full columns (batch 2..4) or .x = own pair (batch 1)
-    struct Piped { uint4 x[NSET]; };
-    const uint2* rem0;
-    const uint4* x0[NSET];   // this lane's 8 X columns of the task's first step, per set
-    const uint32_t* xq0;     // batch 1: this lane's own X pair of the task's first step
-    int last;
-    uint4 xr[XAHEAD][NSET];
-    f32x4_t acc[NSET];
-
-    __device__ __forceinline__ void xload(uint4 (&dst)[NSET], int t) const {
-        t = t < last ? t : last;
-#pragma unroll
-        for (int q = 0; q < NSET; ++q) dst[q] = x0[q][(size_t)t * (kStepCols / 8)];
-    }
-    __device__ __forceinline__ void prime() {
-        if (PIPED) {
-#pragma unroll
-            for (int i = 0; i < XAHEAD; ++i) xload(xr[i], i);
-        }
-    }
-    __device__ __forceinline__ void load(Slot& s, int t) const {
-        t = t < last ? t : last;
-        s.rem = rem0[(size_t)t * kLanes];
-        if (QUARTER) s.x.x = xq0[(size_t)t * (kStepCols / 2)];
-        else if (!PIPED) s.x = x0[0][(size_t)t * (kStepCols / 8)];
-    }
-    __device__ __forceinline__ Piped take(const Slot& s, int i, int t) {
-        Piped p;
-        if (QUARTER) {
-            p.x[0] = make_uint4(s.x.x, quad_bcast<1>(s.x.x), quad_bcast<2>(s.x.x), quad_bcast<3>(s.x.x));
-        } else if (!PIPED) {
-            p.x[0] = s.x;
-        } else {
-#pragma unroll
-            for (int q = 0; q < NSET; ++q) p.x[q] = xr[i % XAHEAD][q];
-            xload(xr[i % XAHEAD], t + XAHEAD);
-        }
-        return p;
-    }
-    __device__ __forceinline__ void use(const Piped& s, int, const uint32_t (&w)[4]) {
-        const bf16x4_t a01 = __builtin_bit_cast(bf16x4_t, make_uint2(w[0], w[1]));
-        const bf16x4_t a23 = __builtin_bit_cast(bf16x4_t, make_uint2(w[2], w[3]));
-#pragma unroll
-        for (int q = 0; q < NSET; ++q) {
-            const bf16x4_t b01 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].x, s.x[q].y));
-            const bf16x4_t b23 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].z, s.x[q].w));
-            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a01, b01, acc[q], 0, 0, 0);
-            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a23, b23, acc[q], 0, 0, 0);
-        }
-    }
-};
-
-struct TaskId { int k, c, t0, t1; };
-
-__device__ __forceinline__ TaskId task_of(const Shape& s, int kc) {
-    TaskId id;
-    id.k = kc / s.nc;
-    id.c = kc % s.nc;
-    id.t0 = (s.steps * id.c) / s.nc;
-    id.t1 = (s.steps * (id.c + 1)) / s.nc;
-    return id;
-}
-
-// ------------------------------------------------------------------ decode to BF16
-template <int NW>
-__global__ __launch_bounds__(NW * kLanes)
-void huffman_decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
-                           uint16_t* __restrict__ Y, const uint32_t* __restrict__ offsets,
-                           const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
-    __shared__ __align__(4096) uint32_t rings[NW][kRingWords];
-    __shared__ uint32_t lut[kTableEntries];
-    load_table(lut, table);
-    __syncthreads();
-
-    const int lane = threadIdx.x & (kLanes - 1);
-    const int wave = (int)uniform(threadIdx.x / kLanes);
-    const int G = s.M / kGroupRows;
-    const int per_group = s.split_k * s.nc;
-    const long long ntasks = (long long)G * per_group;
-    const long long task = (long long)blockIdx.x * NW + wave;
-    if (task >= ntasks) return;
-    const int g = (int)(task / per_group);
-    const TaskId id = task_of(s, (int)(task % per_group));
-
-    HuffCursor cur;
-    cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
-    const int K = s.Ks * s.split_k;
-    StorePolicy pol;
-    pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
-    pol.yp = Y + (size_t)(kGroupRows * g + (lane & 3)) * K + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols;
-    pol.last = id.t1 - id.t0 - 1;
-    if (header_has_esc(header)) run_task<true>(cur, lut, pol, id.t1 - id.t0);
-    else run_task<false>(cur, lut, pol, id.t1 - id.t0);
-}
-
-// ------------------------------------------------------------------ fused decode + GEMV
-// Block = NW wavefronts.  The split_k*nc tasks of one row group are spread over
-// P = min(split_k*nc, NW) wavefronts of the same block (a wavefront loops when there
-// are more tasks than that), so the sum over splits and chunks never leaves the block.
-// register budget: at least this many wavefronts per SIMD must stay resident
-constexpr int min_waves(int bs) { return bs <= 1 ? 6 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
-
-template <int BS, int NW>
-__global__ __launch_bounds__(NW * kLanes, min_waves(BS))
-void gemv_huffman_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
-                         const uint16_t* __restrict__ X, uint16_t* __restrict__ Y,
-                         const uint32_t* __restrict__ offsets, const uint32_t* __restrict__ table,
-                         const uint8_t* __restrict__ header, Shape s, int P, int groups_per_block) {
-    // The partial sums reuse the rings once every task of the block is done.
-    __shared__ __align__(4096) uint32_t rings[NW][kRingWords];
-    __shared__ uint32_t lut[kTableEntries];
-    load_table(lut, table);
-    __syncthreads();
-
-    const int lane = threadIdx.x & (kLanes - 1);
-    const int wave = (int)uniform(threadIdx.x / kLanes);
-    const int G = s.M / kGroupRows;
-    const int per_group = s.split_k * s.nc;
-    const int rg = wave / P, p = wave % P;
-    const int g = blockIdx.x * groups_per_block + rg;
-    const bool active = rg < groups_per_block && g < G;
-    const int K = s.Ks * s.split_k;
-    const bool has_esc = header_has_esc(header);
-
-    MfmaPolicy<BS> pol;
-    constexpr int NSET = MfmaPolicy<BS>::NSET;
-#pragma unroll
-    for (int q = 0; q < NSET; ++q) pol.acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    if (active) {
-        for (int kc = p; kc < per_group; kc += P) {
-            const TaskId id = task_of(s, kc);
-            HuffCursor cur;
-            cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
-            pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
-#pragma unroll
-            for (int q = 0; q < NSET; ++q) {
-                const int batch = (lane & 3) + 4 * q;
-                pol.x0[q] = (const uint4*)(X + (size_t)(batch < BS ? batch : 0) * K + (size_t)id.k * s.Ks
-                                           + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols);
-            }
-            pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
-            pol.last = id.t1 - id.t0 - 1;
-            if (has_esc) run_task<true>(cur, lut, pol, id.t1 - id.t0);
-            else run_task<false>(cur, lut, pol, id.t1 - id.t0);
-        }
-        // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
-#pragma unroll
-        for (int q = 0; q < NSET; ++q) {
-#pragma unroll
-            for (int i = 0; i < kGroupRows; ++i) {
-                float a = pol.acc[q][i];
-                a += __shfl_xor(a, 4);
-                a += __shfl_xor(a, 8);
-                a += __shfl_xor(a, 16);
-                a += __shfl_xor(a, 32);
-                pol.acc[q][i] = a;
-            }
-        }
-    }
-    __syncthreads();                       // every wavefront has finished reading its ring
-    float* mine = (float*)rings[wave];     // partial sums: [set][row][batch lane]
-    if (active && lane < 4) {
-#pragma unroll
-        for (int q = 0; q < NSET; ++q)
-#pragma unroll
-            for (int i = 0; i < kGroupRows; ++i) mine[(q * kGroupRows + i) * 4 + lane] = pol.acc[q][i];
-    }
-    __syncthreads();
-    if (active && p == 0 && lane < 4) {
-#pragma unroll
-        for (int q = 0; q < NSET; ++q) {
-            const int batch = lane + 4 * q;
-            if (batch < BS) {
-#pragma unroll
-                for (int i = 0; i < kGroupRows; ++i) {
-                    float a = 0.f;
-                    for (int w = 0; w < P; ++w) a += ((const float*)rings[rg * P + w])[(q * kGroupRows + i) * 4 + lane];
-                    Y[(size_t)batch * s.M + kGroupRows * g + i] = f32_to_bf16_rne(a);
-                }
-            }
-        }
-    }
-}
 
 // ------------------------------------------------------------------ encoder
 // One wavefront per task: every lane packs its own codes into its own column of the
@@ -399,22 +89,6 @@ void huffman_encode_kernel(const uint8_t* __restrict__ data, const uint32_t* __r
 
 using namespace bhi;
 
-static int check_shape(int split_k, int M, int Ks, int64_t exp_words, int64_t lut1_bytes, Shape* s) {
-    if (split_k < 1 || M < kGroupRows || M % kGroupRows != 0 || Ks < kStepCols || Ks % kStepCols != 0)
-        return bhi_fail(BHI_EINVAL, "need split_k >= 1, M a multiple of 4 and Ks a multiple of 128");
-    if (lut1_bytes != (int64_t)kTableEntries * 4)
-        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 4096 four-byte pair entries");
-    if (exp_words < kTailPadWords || exp_words >= ((int64_t)1 << 32))
-        return bhi_fail(BHI_EINVAL, "exponent stream size out of range");
-    s->M = M; s->Ks = Ks; s->split_k = split_k;
-    s->nc = chunks_per_group(M, Ks, split_k);
-    s->steps = Ks / kStepCols;
-    if ((s->steps + s->nc - 1) / s->nc > kMaxTaskSteps)
-        return bhi_fail(BHI_ELAYOUT, "more than 128 steps per task");
-    s->total_words = (uint32_t)(exp_words - kTailPadWords);
-    return 0;
-}
-
 extern "C" int bhi_huffman_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
                                   void* Y, const void* offsets,
                                   const void* LUT1, int64_t lut1_bytes,
@@ -422,36 +96,11 @@ extern "C" int bhi_huffman_decode(const void* A_rem, const void* A_exp, int64_t 
                                   int split_k, int M, int Ks, void* stream) {
     if (!A_rem || !A_exp || !Y || !offsets || !LUT1 || !code_lengths) return bhi_fail(BHI_EINVAL, "null pointer");
     Shape s;
-    if (int rc = check_shape(split_k, M, Ks, exp_words, lut1_bytes, &s)) return rc;
-    constexpr int NW = 4;
-    long long ntasks = (long long)(M / kGroupRows) * split_k * s.nc;
-    unsigned grid = (unsigned)((ntasks + NW - 1) / NW);
-    hipLaunchKernelGGL(huffman_decode_kernel<NW>, dim3(grid), dim3(NW * kLanes), 0, (hipStream_t)stream,
-                       (const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
-                       (const uint32_t*)LUT1, (const uint8_t*)code_lengths, s);
+    if (lut1_bytes != (int64_t)kTableEntries * 4)
+        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 4096 four-byte pair entries");
+    if (int rc = check_shape(split_k, M, Ks, exp_words, &s)) return rc;
+    launch_decode<HuffCodec>(A_rem, A_exp, Y, offsets, LUT1, code_lengths, s, (hipStream_t)stream);
     return bhi_launch_status("huffman_decode");
-}
-
-template <int BS>
-static void launch_gemv(const void* A_rem, const void* A_exp, const void* X, void* Y, const void* offsets,
-                        const void* LUT1, const void* header, const Shape& s, hipStream_t stream) {
-    const int per_group = s.split_k * s.nc;
-    const int G = s.M / kGroupRows;
-    // small blocks spread more evenly over the 256 CUs; 8 wavefronts only when one row
-    // group needs more than 4 of them
-    if (false) {
-        constexpr int NW = 4;
-        const int P = per_group, gpb = NW / P;
-        hipLaunchKernelGGL((gemv_huffman_kernel<BS, NW>), dim3((unsigned)((G + gpb - 1) / gpb)), dim3(NW * kLanes), 0, stream,
-                           (const uint8_t*)A_rem, (const uint32_t*)A_exp, (const uint16_t*)X, (uint16_t*)Y,
-                           (const uint32_t*)offsets, (const uint32_t*)LUT1, (const uint8_t*)header, s, P, gpb);
-    } else {
-        constexpr int NW = 8;
-        const int P = per_group < NW ? per_group : NW, gpb = NW / P;
-        hipLaunchKernelGGL((gemv_huffman_kernel<BS, NW>), dim3((unsigned)((G + gpb - 1) / gpb)), dim3(NW * kLanes), 0, stream,
-                           (const uint8_t*)A_rem, (const uint32_t*)A_exp, (const uint16_t*)X, (uint16_t*)Y,
-                           (const uint32_t*)offsets, (const uint32_t*)LUT1, (const uint8_t*)header, s, P, gpb);
-    }
 }
 
 extern "C" int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64_t exp_words,
@@ -463,18 +112,10 @@ extern "C" int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64
     if (batch < 1) return bhi_fail(BHI_EINVAL, "batch must be >= 1");
     if (batch > kMaxBatch) return bhi_fail(BHI_EBATCH, "fused GEMV supports batch <= 8");
     Shape s;
-    if (int rc = check_shape(split_k, M, Ks, exp_words, lut1_bytes, &s)) return rc;
-    hipStream_t st = (hipStream_t)stream;
-    switch (batch) {
-        case 1: launch_gemv<1>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        case 2: launch_gemv<2>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        case 3: launch_gemv<3>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        case 4: launch_gemv<4>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        case 5: launch_gemv<5>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        case 6: launch_gemv<6>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        case 7: launch_gemv<7>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-        default: launch_gemv<8>(A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, st); break;
-    }
+    if (lut1_bytes != (int64_t)kTableEntries * 4)
+        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 4096 four-byte pair entries");
+    if (int rc = check_shape(split_k, M, Ks, exp_words, &s)) return rc;
+    launch_gemv_batch<HuffCodec>(batch, A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, (hipStream_t)stream);
     return bhi_launch_status("gemv_bf16_huffman");
 }
 

@@ -248,6 +248,148 @@ def decode(rem_packed: np.ndarray, exp_words: np.ndarray, offsets: np.ndarray, d
     return rebuild_bf16(rem, exp)
 
 
+# ----------------------------------------------------------------------------- rANS codec
+#
+# Same planes, tasks, lanes, rows and offsets as the Huffman stream; a task block is
+# ``[W rows of 64 words][zero pad]`` with no escape list.  Each lane owns ONE rANS state
+# (64 bit, precision 8, 32-bit renormalisation words), i.e. the reference's state and
+# tables (``src/kernel.cu:652-683``, ``ans.py:6-80``) with a different renormalisation
+# schedule: the decoder looks at its state only after every FOUR symbols (the two halves
+# of a step) and pulls one word when the state has dropped below 2**32.  Decoding is the
+# exact inverse of encoding for any state value, so four symbols may be taken without a
+# refill; the encoder (which runs backwards) emits the low word of its state before a
+# half-step whenever encoding the four symbols would overflow 64 bits or the decoder
+# would see a state below 2**32.  Rows 0 and 1 of a lane are its initial state.
+
+ANS_PRECISION = 8
+ANS_HALF = 4                   # symbols between two refill checks
+ANS_INIT_ROWS = 2
+
+
+def ans_capacity(n_steps: int) -> int:
+    return LANES * (2 * n_steps + ANS_INIT_ROWS) + ALIGN_WORDS
+
+
+def _ans_encode_tasks(sym: np.ndarray, freq: np.ndarray, cum: np.ndarray):
+    """sym: uint8 [nt, ns, 64, 8] -> list of nt uint32 task blocks."""
+    nt, ns = sym.shape[:2]
+    U = np.uint64
+    f_of, c_of = freq.astype(np.uint64), cum.astype(np.uint64)
+    assert (f_of[np.unique(sym)] > 0).all(), "symbol without a frequency"
+    x = np.full((nt, LANES), 1 << 32, dtype=np.uint64)
+    rev = np.zeros((nt, LANES, 2 * ns + ANS_INIT_ROWS), dtype=np.uint32)        # emission order
+    n = np.zeros((nt, LANES), dtype=np.int64)
+    ti, li = np.indices((nt, LANES))
+
+    def emit(mask, value):
+        rev[ti[mask], li[mask], n[mask]] = value[mask].astype(np.uint32)
+        n[mask] += 1
+
+    for t in range(ns - 1, -1, -1):
+        for half in (1, 0):
+            s4 = sym[:, t, :, ANS_HALF * half:ANS_HALF * (half + 1)].astype(np.int64)    # [nt, 64, 4]
+            # would the four symbols fit without a refill?
+            y, fits = x.copy(), x >= U(1 << 32)
+            for j in range(ANS_HALF - 1, -1, -1):
+                f, c = f_of[s4[..., j]], c_of[s4[..., j]]
+                q = y // f
+                fits &= q < U(1 << 56)
+                y = ((q & U((1 << 56) - 1)) << U(8)) + (y % f) + c
+            must = ~fits
+            emit(must, x & U(0xFFFFFFFF))
+            x = np.where(must, x >> U(32), x)
+            for j in range(ANS_HALF - 1, -1, -1):
+                f, c = f_of[s4[..., j]], c_of[s4[..., j]]
+                x = ((x // f) << U(8)) + (x % f) + c
+    every = np.ones((nt, LANES), dtype=bool)
+    emit(every, x >> U(32))
+    emit(every, x & U(0xFFFFFFFF))
+
+    rows = n.max(axis=-1)
+    blocks = []
+    for t in range(nt):
+        W = int(rows[t])
+        total = (W * LANES + ALIGN_WORDS - 1) // ALIGN_WORDS * ALIGN_WORDS
+        blk = np.zeros(total, dtype=np.uint32)
+        lw = np.zeros((LANES, W), dtype=np.uint32)
+        col = np.arange(W)[None, :]
+        src = n[t][:, None] - 1 - col                               # decode order = reverse emission
+        keep = src >= 0
+        lw[keep] = rev[t][np.broadcast_to(np.arange(LANES)[:, None], src.shape)[keep], src[keep]]
+        blk[:W * LANES] = lw.T.reshape(-1)
+        blocks.append(blk)
+    return blocks
+
+
+def _ans_decode_tasks(words: np.ndarray, base: np.ndarray, ns: int, lut: np.ndarray) -> np.ndarray:
+    """Step-by-step model of one wavefront per task.  lut: uint32[256] packed
+    (sym<<24)|(freq<<12)|rem."""
+    nt = len(base)
+    U = np.uint64
+    lanes = np.arange(LANES)
+    w64 = words.astype(np.uint64)
+    lut64 = lut.astype(np.uint64)
+    at = base[:, None] + lanes
+    x = w64[at] | (w64[at + LANES] << U(32))
+    row = np.full((nt, LANES), ANS_INIT_ROWS, dtype=np.int64)
+    out = np.zeros((nt, ns, LANES, LANE_COLS), dtype=np.uint8)
+    limit = len(words) - 1
+    for t in range(ns):
+        for half in (0, 1):
+            for j in range(ANS_HALF):
+                e = lut64[(x & U(0xFF)).astype(np.int64)]
+                out[:, t, :, ANS_HALF * half + j] = (e >> U(24)).astype(np.uint8)
+                x = ((e >> U(12)) & U(0xFFF)) * (x >> U(8)) + (e & U(0xFFF))
+            need = x < U(1 << 32)
+            w = w64[np.minimum(base[:, None] + row * LANES + lanes, limit)]
+            x = np.where(need, (x << U(32)) | w, x)
+            row = row + need
+    return out
+
+
+def encode_ans(bits: np.ndarray, split_k: int, freq: np.ndarray, cum: np.ndarray):
+    """bits: uint16 [M, K] BF16 patterns -> dict(rem, exp, offsets, nc)."""
+    from .planes import split_bf16
+    M, K = bits.shape
+    Ks = K // split_k
+    S, G = Ks // STEP_COLS, M // GROUP_ROWS
+    nc = chunks_per_group(M, Ks, split_k)
+    rem, exp = split_bf16(bits)
+    sym = lane_order(exp, split_k)
+    per_chunk = []
+    for c in range(nc):
+        t0, t1 = chunk_steps(S, nc, c)
+        per_chunk.append(_ans_encode_tasks(sym[:, :, t0:t1].reshape(split_k * G, t1 - t0, LANES, LANE_COLS), freq, cum))
+    offsets = np.zeros((split_k, M), dtype=np.int64)
+    parts, cursor = [], 0
+    for k in range(split_k):
+        for g in range(G):
+            for c in range(nc):
+                blk = per_chunk[c][k * G + g]
+                offsets[k, GROUP_ROWS * g + c] = cursor
+                parts.append(blk)
+                cursor += len(blk)
+    parts.append(np.zeros(TAIL_PAD_WORDS, dtype=np.uint32))
+    return {"rem": pack_rem(rem, split_k), "exp": np.concatenate(parts).view(np.int32),
+            "offsets": offsets.astype(np.int32), "nc": nc}
+
+
+def decode_ans(rem_packed: np.ndarray, exp_words: np.ndarray, offsets: np.ndarray, lut: np.ndarray) -> np.ndarray:
+    """-> uint16 [M, K] BF16 patterns."""
+    from .planes import rebuild_bf16
+    split_k, M, Ks = rem_packed.shape
+    S, G = Ks // STEP_COLS, M // GROUP_ROWS
+    nc = chunks_per_group(M, Ks, split_k)
+    words = exp_words.view(np.uint32)
+    off = offsets.astype(np.int64).reshape(split_k, G, GROUP_ROWS)[:, :, :nc]
+    sym = np.zeros((split_k, G, S, LANES, LANE_COLS), dtype=np.uint8)
+    for c in range(nc):
+        t0, t1 = chunk_steps(S, nc, c)
+        r = _ans_decode_tasks(words, off[:, :, c].reshape(-1), t1 - t0, lut.view(np.uint32))
+        sym[:, :, t0:t1] = r.reshape(split_k, G, t1 - t0, LANES, LANE_COLS)
+    return rebuild_bf16(unpack_rem(rem_packed), lane_order_inverse(sym))
+
+
 # ----------------------------------------------------------------------------- table checks
 
 def check_tables(dec: np.ndarray, enc: np.ndarray) -> None:

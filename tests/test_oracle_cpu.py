@@ -255,3 +255,50 @@ def test_c_abi_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
+
+
+# ----------------------------------------------------------------------------- rANS in the wave64 layout
+
+@pytest.mark.parametrize("kind,M,K,n", [("gauss", 64, 1024, 1), ("t3", 32, 768, 2), ("bits", 16, 384, 1),
+                                        ("special", 32, 512, 1), ("zeros", 8, 384, 1)])
+def test_wave64_ans_round_trip(kind, M, K, n):
+    makers = {"gauss": gaussian_weight, "t3": student_t_weight, "bits": random_bits_weight,
+              "special": special_values_weight, "zeros": lambda M, K, seed=0: torch.zeros(M, K, dtype=torch.bfloat16)}
+    bits = bits_of(makers[kind](M, K, seed=2))
+    _, exp = planes.split_bf16(bits)
+    freq, cum, lut = ref_tables.ans_tables(np.bincount(exp.reshape(-1), minlength=256), 8)
+    enc = wave64.encode_ans(bits, n, freq, cum)
+    assert enc["exp"].dtype == np.int32 and (len(enc["exp"]) - wave64.TAIL_PAD_WORDS) % wave64.ALIGN_WORDS == 0
+    assert np.array_equal(wave64.decode_ans(enc["rem"], enc["exp"], enc["offsets"], lut), bits)
+    # the reference layout with the reference's own schedule gives back the same tensor
+    ref = ref_layout.encode(bits, n, "ans", (freq, cum))
+    assert np.array_equal(ref_layout.decode_ans(ref["rem"], ref["exp"], ref["offsets"], lut), bits)
+
+
+def test_wave64_ans_state_schedule_by_hand():
+    """One lane worked by hand with the tables of ans.py:152 (freq 1:96 2:32 3:32 ...).
+
+    Symbols of the only step: [1,1,1,1 | 1,1,1,1].  Encoder, backwards from x = 2**32:
+    second half: x >= 2**32 and fits -> no word; four pushes of symbol 1 (f=96, c=0):
+    x -> ((x // 96) << 8) + x % 96, four times; first half: same.  The block then holds
+    the final state in rows 1 (high word) and 0 (low word), and the decoder must come
+    back to exactly 2**32 without ever pulling a word."""
+    counts = np.bincount([1, 2, 3, 3, 2, 12, 13, 11, 1, 8, 1, 7, 1, 6, 1, 1], minlength=256)
+    freq, cum, lut = ref_tables.ans_tables(counts, 8)
+    x = 1 << 32
+    for _ in range(8):
+        x = ((x // 96) << 8) + x % 96
+    sym = np.ones((1, 1, wave64.LANES, wave64.LANE_COLS), dtype=np.uint8)
+    blk = wave64._ans_encode_tasks(sym, freq, cum)[0]
+    assert len(blk) == 2 * wave64.LANES
+    assert (blk[:wave64.LANES] == (x & 0xFFFFFFFF)).all() and (blk[wave64.LANES:] == (x >> 32)).all()
+    words = np.concatenate([blk, np.zeros(256, dtype=np.uint32)])
+    out = wave64._ans_decode_tasks(words, np.array([0]), 1, lut.view(np.uint32))
+    assert (out == 1).all()
+
+
+def test_ans_capacity_matches_library():
+    from bf16_huffman_infer_amd import _lib
+    lib = _lib.load()
+    for ns in (1, 4, 28, 37, 128):
+        assert lib.bhi_ans_encode_capacity(ns) == wave64.ans_capacity(ns)
