@@ -1,0 +1,223 @@
+"""Greedy decode of a random-init Qwen3-8B-shaped decoder, raw BF16 against compressed.
+
+The decoder below is the Qwen3 architecture (RMSNorm, grouped-query attention with
+per-head q/k RMSNorm and rotary embedding, SwiGLU MLP, untied lm_head) written so that one
+decode step is a pure function of device tensors: the position, the current token and the
+KV cache live on the GPU and the step updates them itself, so the step can be recorded
+into one HIP graph and replayed back to back with no host interaction.  Every projection
+is an ``nn.Linear``: ``convert_all_linear`` swaps them for compressed modules in place.
+
+Protocol (bs=1): 16 random prompt ids, then 256 greedy tokens, static KV cache of 1024
+slots; tokens/s is taken over the 256 decode steps (prompt excluded), best of 3.
+
+Prints one JSON line with raw and compressed tokens/s, their ratio, the footprints from
+``get_model_size`` and whether the generated ids agree (they must: decoding is lossless
+and both paths accumulate in fp32, but the summation order differs, so agreement is
+reported as the length of the common prefix rather than asserted).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+class Config:
+    def __init__(self, layers=36, hidden=4096, intermediate=12288, q_heads=32, kv_heads=8, head_dim=128,
+                 vocab=151936, max_len=1024, rope_theta=1e6, eps=1e-6):
+        self.__dict__.update(locals())
+        del self.__dict__["self"]
+
+
+def rms_norm(x, weight, eps):
+    return F.rms_norm(x, (x.shape[-1],), weight, eps)
+
+
+class Block(nn.Module):
+    def __init__(self, c: Config):
+        super().__init__()
+        self.c = c
+        self.q_proj = nn.Linear(c.hidden, c.q_heads * c.head_dim, bias=False)
+        self.k_proj = nn.Linear(c.hidden, c.kv_heads * c.head_dim, bias=False)
+        self.v_proj = nn.Linear(c.hidden, c.kv_heads * c.head_dim, bias=False)
+        self.o_proj = nn.Linear(c.q_heads * c.head_dim, c.hidden, bias=False)
+        self.gate_proj = nn.Linear(c.hidden, c.intermediate, bias=False)
+        self.up_proj = nn.Linear(c.hidden, c.intermediate, bias=False)
+        self.down_proj = nn.Linear(c.intermediate, c.hidden, bias=False)
+        # per-head RMSNorm weights of q and k, stacked so that both are normalised and
+        # rotated in one pass: [q_heads + kv_heads, head_dim]
+        self.qk_norm = nn.Parameter(torch.ones(c.q_heads + c.kv_heads, c.head_dim))
+        self.input_norm = nn.Parameter(torch.ones(c.hidden))
+        self.post_norm = nn.Parameter(torch.ones(c.hidden))
+
+    def forward(self, x, pos, cos, sin, visible, k_cache, v_cache):
+        c = self.c
+        h = rms_norm(x, self.input_norm, c.eps)
+        qk = torch.cat((self.q_proj(h), self.k_proj(h)), -1).view(c.q_heads + c.kv_heads, c.head_dim)
+        v = self.v_proj(h).view(c.kv_heads, 1, c.head_dim)
+        qk = rope(F.rms_norm(qk, (c.head_dim,), None, c.eps) * self.qk_norm, cos, sin)
+        q, k = qk[:c.q_heads], qk[c.q_heads:]
+        k_cache.index_copy_(1, pos, k[:, None, :])                      # [kv, max_len, d]
+        v_cache.index_copy_(1, pos, v)
+        a = F.scaled_dot_product_attention(q[None, :, None, :], k_cache[None], v_cache[None],
+                                           attn_mask=visible, enable_gqa=True)      # [1, q, 1, d]
+        x = x + self.o_proj(a.reshape(1, c.q_heads * c.head_dim))
+        h = rms_norm(x, self.post_norm, c.eps)
+        return x + self.down_proj(F.silu(self.gate_proj(h)) * self.up_proj(h))
+
+
+def rope(x, cos, sin):
+    """x [heads, d] (bf16), cos/sin [1, d/2] (fp32): rotate-half convention."""
+    half = x.shape[-1] // 2
+    x1, x2 = x[..., :half].float(), x[..., half:].float()
+    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), -1).to(x.dtype)
+
+
+class Decoder(nn.Module):
+    def __init__(self, c: Config):
+        super().__init__()
+        self.c = c
+        self.embed = nn.Embedding(c.vocab, c.hidden)
+        self.blocks = nn.ModuleList(Block(c) for _ in range(c.layers))
+        self.norm = nn.Parameter(torch.ones(c.hidden))
+        self.lm_head = nn.Linear(c.hidden, c.vocab, bias=False)
+
+    def init_state(self, device):
+        c = self.c
+        inv = 1.0 / (c.rope_theta ** (torch.arange(0, c.head_dim, 2, device=device).float() / c.head_dim))
+        ang = torch.arange(c.max_len, device=device).float()[:, None] * inv[None, :]
+        self.cos, self.sin = ang.cos(), ang.sin()                        # [max_len, d/2]
+        self.k_cache = torch.zeros(c.layers, c.kv_heads, c.max_len, c.head_dim, dtype=torch.bfloat16, device=device)
+        self.v_cache = torch.zeros_like(self.k_cache)
+        self.slots = torch.arange(c.max_len, device=device)
+        self.pos = torch.zeros(1, dtype=torch.int64, device=device)
+        self.token = torch.zeros(1, dtype=torch.int64, device=device)
+        self.out = torch.zeros(c.max_len, dtype=torch.int64, device=device)
+
+    def step(self):
+        """One token: consumes ``token`` at ``pos``, stores the greedy next token in ``token``
+        and ``out[pos]``, advances ``pos``.  Device tensors only."""
+        pos = self.pos
+        x = self.embed(self.token)                                       # [1, hidden]
+        cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
+        visible = (self.slots <= pos).view(1, 1, 1, -1)
+        for i, blk in enumerate(self.blocks):
+            x = blk(x, pos, cos, sin, visible, self.k_cache[i], self.v_cache[i])
+        logits = self.lm_head(rms_norm(x, self.norm, self.c.eps))
+        nxt = logits.argmax(-1)
+        self.out.index_copy_(0, pos, nxt)
+        self.token.copy_(nxt)
+        self.pos.add_(1).clamp_(max=self.c.max_len - 1)                  # a replay past the cache stays in range
+        return logits
+
+
+def build(c: Config, device, seed=0):
+    """Random-init on the device: N(0, 0.02) for every matrix, ones for the norms."""
+    with torch.device("meta"):
+        model = Decoder(c)
+    model = model.to_empty(device=device).bfloat16()
+    g = torch.Generator(device=device).manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if not name.endswith("norm"):
+                p.copy_((torch.randn(p.shape, generator=g, device=device) * 0.02).bfloat16())
+            else:
+                p.fill_(1.0)
+    model.eval()
+    model.init_state(device)
+    return model
+
+
+def generate(model: Decoder, prompt: torch.Tensor, new_tokens: int, graphed=True):
+    """Returns (ids of the new tokens, seconds spent on the ``new_tokens`` decode steps)."""
+    from bf16_huffman_infer_amd.cudagraph_utils import GraphedCallable
+    c = model.c
+    assert len(prompt) + new_tokens <= c.max_len
+    step = getattr(model, "_graph", None)
+    if graphed and step is None:
+        model.pos.fill_(c.max_len - 1)                                   # record at the last slot
+        step = model._graph = GraphedCallable(lambda: model.step(), ())
+    run = step.replay if graphed else (lambda: model.step())
+    with torch.no_grad():
+        model.k_cache.zero_(); model.v_cache.zero_(); model.pos.zero_()
+        for t in prompt.tolist():                                        # prompt: one token at a time
+            model.token.fill_(t)
+            run()
+        first = int(model.pos.item())                                    # == len(prompt); token now holds the first new id
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(new_tokens):
+            run()
+        stop.record()
+        torch.cuda.synchronize()
+    ids = model.out[first - 1:first - 1 + new_tokens + 1].clone()        # out[p] = token chosen after consuming position p
+    return ids, start.elapsed_time(stop) * 1e-3
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--tokens", type=int, default=256)
+    ap.add_argument("--prompt", type=int, default=16)
+    ap.add_argument("--algo", default="smallest", choices=["huffman", "ans", "smallest"])
+    ap.add_argument("--repeats", type=int, default=3)
+    ap.add_argument("--small", action="store_true", help="tiny shapes (smoke run)")
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        sys.exit("bench_decode.py needs a GPU")
+    from bf16_huffman_infer_amd import _lib, convert_all_linear, get_model_size
+    _lib.load()
+    device = torch.device("cuda", 0)
+    c = Config(layers=args.layers)
+    if args.small:
+        c = Config(layers=2, hidden=512, intermediate=1024, q_heads=4, kv_heads=2, head_dim=128, vocab=4096)
+    model = build(c, device)
+    g = torch.Generator().manual_seed(1)
+    prompt = torch.randint(0, c.vocab, (args.prompt,), generator=g)
+
+    def best(model):
+        runs = [generate(model, prompt, args.tokens) for _ in range(args.repeats)]
+        assert all(torch.equal(runs[0][0], r[0]) for r in runs), "generation is not reproducible"
+        return runs[0][0], min(r[1] for r in runs)
+
+    raw_size = get_model_size(model)
+    raw_ids, raw_s = best(model)
+    print(f"raw BF16: {args.tokens / raw_s:.1f} tok/s, {raw_size / 2**30:.2f} GiB", flush=True)
+
+    del model._graph
+    t0 = time.time()
+    convert_all_linear(model, min_out_features=0, progress=False, algo=args.algo)
+    model.to(device)
+    convert_s = time.time() - t0
+    kinds = {}
+    for m in model.modules():
+        if type(m).__name__ in ("HuffmanWeight", "ANSWeight"):
+            kinds[type(m).__name__] = kinds.get(type(m).__name__, 0) + 1
+    new_size = get_model_size(model)
+    new_ids, new_s = best(model)
+    same = int((raw_ids == new_ids).long().cumprod(0).sum().item())
+    print(json.dumps({
+        "workload": f"Qwen3-8B-shaped decoder ({c.layers} layers, hidden {c.hidden}, intermediate {c.intermediate}, "
+                    f"{c.q_heads}/{c.kv_heads} heads, vocab {c.vocab}), random init N(0,0.02), bs=1, "
+                    f"{args.prompt}-token prompt, {args.tokens} greedy tokens, static KV {c.max_len}, hipGraph step",
+        "algo": args.algo, "modules": kinds,
+        "raw_tokens_per_s": round(args.tokens / raw_s, 2), "compressed_tokens_per_s": round(args.tokens / new_s, 2),
+        "compressed_over_raw": round(raw_s / new_s, 4),
+        "raw_ms_per_token": round(raw_s / args.tokens * 1e3, 4), "compressed_ms_per_token": round(new_s / args.tokens * 1e3, 4),
+        "raw_gib": round(raw_size / 2**30, 3), "compressed_gib": round(new_size / 2**30, 3),
+        "footprint_ratio": round(new_size / raw_size, 4),
+        "common_prefix_tokens": same, "tokens": args.tokens + 1, "convert_seconds": round(convert_s, 1),
+    }))
+
+
+if __name__ == "__main__":
+    main()

@@ -8,3 +8,4 @@ Drop-in for the Python surface of lszxb/bf16_huffman_infer::
 from .functional import *  # noqa: F401,F403
 from .functional import mv_ans, mv_huffman  # noqa: F401
 from .utils import get_model_size  # noqa: F401
+from .cudagraph_utils import get_graphed_model  # noqa: F401,E402

@@ -1,0 +1,143 @@
+"""HIP-graph capture of the one-token decode step.
+
+Counterpart of the reference's ``bf16_huffman_infer/cudagraph_utils.py``
+(``apply_graphed`` ``:11-80``, ``get_graphed_model`` ``:83-86``): the single-token forward of
+a causal LM with a static KV cache is recorded once and replayed per token, prefill runs
+eagerly, and ``generate`` is patched to reuse the one cache.  The reference goes through
+``torch.cuda.make_graphed_callables``; here the step is recorded straight into a
+``torch.cuda.CUDAGraph`` (a hipGraph on ROCm) over static input buffers, because the step
+runs under ``no_grad`` and needs none of the autograd plumbing -- and because the fused
+kernels are launched through the C ABI on the capturing stream, which is all a capture
+needs from them.
+
+:class:`GraphedCallable` is the model-independent part: any function of tensors whose
+launches stay on the current stream can be recorded with it.
+"""
+from typing import Callable, Sequence
+
+import torch
+from torch import nn
+
+from .utils import shallow_copy_model
+
+__all__ = ["GraphedCallable", "apply_graphed", "get_graphed_model"]
+
+
+class GraphedCallable:
+    """``fn(*tensors) -> tensor(s)`` recorded into one graph.
+
+    ``sample_args`` fix shapes, dtypes and devices; they become the static input buffers.
+    Calling the object copies the arguments into those buffers, replays the graph and
+    returns the static output tensor(s) -- the same storage on every call, so a caller
+    that keeps results across calls must clone them.
+
+    No memset is recorded by this class itself; ``fn`` must not allocate-and-zero through
+    paths that record memset nodes (use ``tensor.zero_()``, which is a fill kernel).
+    """
+
+    def __init__(self, fn: Callable, sample_args: Sequence[torch.Tensor], warmup: int = 3):
+        self.static_inputs = [a.clone() for a in sample_args]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(warmup):
+                fn(*self.static_inputs)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(self.graph):
+            self.static_outputs = fn(*self.static_inputs)
+
+    def __call__(self, *args: torch.Tensor):
+        assert len(args) == len(self.static_inputs)
+        for dst, src in zip(self.static_inputs, args):
+            if src is not dst:
+                dst.copy_(src)
+        self.graph.replay()
+        return self.static_outputs
+
+    def replay(self):
+        """Replay on the current contents of the static inputs."""
+        self.graph.replay()
+        return self.static_outputs
+
+
+def _max_cache_len(cache) -> int:
+    for name in ("get_max_length", "get_max_cache_shape"):
+        fn = getattr(cache, name, None)
+        if fn is not None:
+            return int(fn())
+    return int(cache.max_cache_len)
+
+
+def apply_graphed(model, cache, replace_generate: bool = True) -> None:
+    """Patch ``model.forward`` in place: one-token calls replay a graph, longer calls
+    (prefill) run eagerly; both write into ``cache``.  With ``replace_generate`` the
+    model's ``generate`` resets and passes that cache on every call
+    (reference ``cudagraph_utils.py:11-80``)."""
+    from transformers.modeling_outputs import CausalLMOutputWithPast
+
+    _old_forward = model.forward
+    device = model.device
+    dtype = model.dtype
+    max_len = _max_cache_len(cache)
+    key_index = torch.arange(max_len, device=device)
+
+    def _forward(input_ids, attention_mask, position_ids, cache_position):
+        with torch.no_grad():
+            return _old_forward(
+                input_ids=input_ids,
+                attention_mask=attention_mask,
+                position_ids=position_ids,
+                past_key_values=cache,
+                output_attentions=False,
+                output_hidden_states=False,
+                use_cache=True,
+                cache_position=cache_position,
+                return_dict=True,
+            ).logits
+
+    def _step(input_ids, cache_position):
+        # the one-token step sees every cache slot up to its own position; an additive
+        # mask over the whole static cache keeps every shape independent of the position
+        visible = key_index[None, None, None, :] <= cache_position.view(1, 1, 1, 1)
+        mask = torch.zeros(1, 1, 1, max_len, dtype=dtype, device=device).masked_fill_(~visible, float("-inf"))
+        return _forward(input_ids, mask, cache_position.view(1, 1), cache_position)
+
+    # recorded at the last cache slot so that the warm-up runs do not disturb a prompt
+    step = GraphedCallable(_step, (
+        torch.zeros(1, 1, dtype=torch.int64, device=device),
+        torch.tensor([max_len - 1], dtype=torch.int64, device=device),
+    ))
+    cache.reset()
+
+    def forward(input_ids=None, attention_mask=None, position_ids=None, cache_position=None, **unused):
+        # `unused` swallows what generate() passes besides (past_key_values, use_cache, ...):
+        # the cache is the one given to apply_graphed, outputs are logits only
+        if cache_position is None:
+            start = cache.get_seq_length()
+            cache_position = torch.arange(start, start + input_ids.shape[1], device=input_ids.device)
+        if input_ids.shape[0] == 1 and input_ids.shape[1] == 1:
+            logits = step(input_ids, cache_position.view(1)).clone()
+        else:
+            logits = _forward(input_ids, attention_mask, position_ids, cache_position)
+        return CausalLMOutputWithPast(logits=logits, past_key_values=cache)
+
+    model.forward = forward
+
+    if replace_generate:
+        _old_generate = model.generate
+
+        def generate(*args, **kwargs):
+            cache.reset()
+            return _old_generate(*args, past_key_values=cache, disable_compile=True, **kwargs)
+
+        model.generate = generate
+
+
+def get_graphed_model(model: nn.Module, cache) -> nn.Module:
+    """A copy of ``model`` that shares its weights and decodes through a recorded graph
+    (reference ``cudagraph_utils.py:83-86``)."""
+    graphed_model = shallow_copy_model(model)
+    apply_graphed(graphed_model, cache)
+    return graphed_model
