@@ -88,7 +88,7 @@ def time_launches(fn, n, warmup, launches_per_graph=1):
     return start.elapsed_time(stop) * 1e-3 / (replays * launches_per_graph)
 
 
-def cpu_baseline(rows=4096, K=3584, reps=3):
+def cpu_baseline(rows=18944, K=3584, reps=5):
     """Reference layout + reference decoder (numpy) + host matmul on a slice of gate_proj."""
     import numpy as np
     from oracle import planes, ref_layout, ref_tables
@@ -115,9 +115,9 @@ def cpu_baseline(rows=4096, K=3584, reps=3):
     total, t_dec, t_mm = times[len(times) // 2]
     return {
         "value": round(nbytes / total / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"first {rows} rows of gate_proj ({rows}x{K}), reference layout; numpy decode {t_dec:.2f}s "
-                  f"(1 thread) + torch matmul {t_mm * 1e3:.1f}ms ({torch.get_num_threads()} threads); "
-                  f"os.cpu_count()={os.cpu_count()}",
+        "sample": f"gate_proj ({rows}x{K}) of the workload, reference layout, median of {reps} passes "
+                  f"({sum(t[0] for t in times):.1f}s of CPU work); numpy decode {t_dec:.2f}s (1 thread) + torch matmul "
+                  f"{t_mm * 1e3:.1f}ms ({torch.get_num_threads()} threads); os.cpu_count()={os.cpu_count()}",
     }
 
 
@@ -202,8 +202,8 @@ def main():
             sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),
         "block_steps_per_s": round(1.0 / sec, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
-        "roofline": {"bound": "hbm", "kernel": f"gemv_huffman_kernel<{bs}> 18944x3584" if args.algo == "huffman"
-                     else f"gemv_ans_kernel<{bs}> 18944x3584",
+        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{'HuffCodec' if args.algo == 'huffman' else 'AnsCodec'}, {bs}, 8> "
+                               f"18944x3584",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.algo, bs)),

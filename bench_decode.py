@@ -81,6 +81,20 @@ def rope(x, cos, sin):
     return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), -1).to(x.dtype)
 
 
+def greedy(logits):
+    """argmax over the vocabulary in two small stages.  A single reduction over 150k values
+    makes torch use its multi-block reduce, whose semaphore buffer is cleared by a memset
+    node when recorded into a graph; two stages of at most a few thousand values each stay
+    within one block per output and record kernels only."""
+    n = logits.shape[-1]
+    width = 256
+    pad = (-n) % width
+    v = F.pad(logits.view(-1), (0, pad), value=float("-inf")).view(-1, width)
+    best, col = v.max(-1)
+    row = best.argmax(0, keepdim=True)
+    return row * width + col.index_select(0, row)
+
+
 class Decoder(nn.Module):
     def __init__(self, c: Config):
         super().__init__()
@@ -106,13 +120,13 @@ class Decoder(nn.Module):
         """One token: consumes ``token`` at ``pos``, stores the greedy next token in ``token``
         and ``out[pos]``, advances ``pos``.  Device tensors only."""
         pos = self.pos
-        x = self.embed(self.token)                                       # [1, hidden]
+        x = self.embed(self.token.clamp(0, self.c.vocab - 1))            # [1, hidden]
         cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
         visible = (self.slots <= pos).view(1, 1, 1, -1)
         for i, blk in enumerate(self.blocks):
             x = blk(x, pos, cos, sin, visible, self.k_cache[i], self.v_cache[i])
         logits = self.lm_head(rms_norm(x, self.norm, self.c.eps))
-        nxt = logits.argmax(-1)
+        nxt = greedy(logits)
         self.out.index_copy_(0, pos, nxt)
         self.token.copy_(nxt)
         self.pos.add_(1).clamp_(max=self.c.max_len - 1)                  # a replay past the cache stays in range
