@@ -29,7 +29,10 @@ constexpr int kMaxBatch = 8;
 constexpr int kAnsPrecision = 8;
 constexpr int kAlignWords = 4;
 constexpr int kTailPadWords = 2048;
-constexpr int kTargetTasks = 6144;      // wavefronts kept resident: 256 CUs x 4 SIMDs x 6
+#ifndef BHI_TARGET_TASKS
+#define BHI_TARGET_TASKS 6144
+#endif
+constexpr int kTargetTasks = BHI_TARGET_TASKS;      // wavefronts kept resident: 256 CUs x 4 SIMDs x 6
 constexpr int kMinChunkSteps = 4;
 constexpr int kMaxChunks = 4;
 constexpr int kMaxTaskSteps = 128;
@@ -83,20 +86,26 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
 }
 
 // A task is processed in segments of kSegSteps steps; the global loads of a segment
-// (all unconditional, with clamped indices) are issued one segment ahead of their use.
+// (all unconditional, with clamped indices) are issued back to back before it is decoded.
 // VMEM loads complete in issue order, so a load issued on demand inside a segment would
 // make its wait drain the whole queue.
 //
 // Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each,
 // the ring is aligned to its 4 KB size so that a slot address is an AND and an OR).
 // Row r lives in slot r % kRingRows.  Lanes sit at different rows, yet row r of lane l
-// is always in bank l % 32: window reads are conflict free.  Every segment prefetches the next kSegRows rows and commits them to
-// the ring once the previous segment is decoded; a lane whose window is not staged (a
-// cheap per-step test) reads it from global memory instead.
-constexpr bool kPipelined = false;
-constexpr int kSegSteps = 8;
-constexpr int kRingRows = 16;
-constexpr int kSegRows = 8;          // rows prefetched per segment = the most a lane can consume in one
+// is always in bank l % 32: window reads are conflict free.  Every segment prefetches
+// the next kSegRows rows and commits them to the ring before it is decoded; a lane whose window is not staged (a cheap per-step
+// test) reads it from global memory instead.
+#ifndef BHI_SEG_STEPS
+#define BHI_SEG_STEPS 8
+#define BHI_SEG_ROWS 8
+#endif
+constexpr int kSegSteps = BHI_SEG_STEPS;
+#ifndef BHI_RING_ROWS
+#define BHI_RING_ROWS 16
+#endif
+constexpr int kRingRows = BHI_RING_ROWS;
+constexpr int kSegRows = BHI_SEG_ROWS;          // rows prefetched per segment
 constexpr int kRingSlots = kRingRows;
 constexpr int kRingWords = kRingSlots * kLanes;
 

@@ -25,14 +25,13 @@ struct Shape {
     uint32_t total_words;
 };
 
-// Runs one task as a two-stage software pipeline over segments of kSegSteps steps: while
-// segment s is decoded, the loads of segment s+1 (operand slots and the next exponent
-// rows) are in flight.  A policy supplies the operands that travel with the exponent
-// stream: `Slot` holds what is loaded per step (`load(slot, t)`, t clamped by the
-// policy); `take(...)` hands out what the policy pipelines on its own inside the
-// compute phase; `use(...)` receives the lane's four rebuilt BF16 pairs (columns 0..7
-// of its row in step t).  Every global load is unconditional, so the compiler can
-// count outstanding loads and wait for exactly the ones a step needs.
+// Runs one task in segments of kSegSteps steps: load phase (every global load of the
+// segment, unconditional), then decode.  A policy supplies the operands that travel with
+// the exponent stream: `Slot` holds what is loaded per step (`load(slot, t)`, t clamped by
+// the policy); `take(...)` hands out what the policy pipelines on its own inside the
+// compute phase; `use(...)` receives the lane's four rebuilt BF16 pairs (columns 0..7 of
+// its row in step t).  Because every load is unconditional the compiler can count the
+// outstanding ones and make each step wait for exactly its own operands.
 template <class Policy>
 __device__ __forceinline__ void load_segment(const Policy& pol, typename Policy::Slot (&slot)[kSegSteps], int t0) {
 #pragma unroll
@@ -62,33 +61,15 @@ __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut,
 template <bool HAS_ESC, class Cursor, class Policy>
 __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns) {
     pol.prime();
-    if (kPipelined) {
-        typename Policy::Slot sa[kSegSteps], sb[kSegSteps];
-        uint32_t ra[kSegRows], rb[kSegRows];
-        load_segment(pol, sa, 0);
-        cur.prime();
-        cur.start();
-        for (int seg = 0; seg < ns; seg += 2 * kSegSteps) {
-            cur.prefetch(rb);
-            load_segment(pol, sb, seg + kSegSteps);
-            decode_segment<HAS_ESC>(cur, lut, pol, sa, seg, ns);
-            cur.commit(rb);
-            cur.prefetch(ra);
-            load_segment(pol, sa, seg + 2 * kSegSteps);
-            decode_segment<HAS_ESC>(cur, lut, pol, sb, seg + kSegSteps, ns);
-            cur.commit(ra);
-        }
-    } else {
-        cur.prime();
-        cur.start();
-        for (int seg = 0; seg < ns; seg += kSegSteps) {
-            typename Policy::Slot slot[kSegSteps];
-            uint32_t rows[kSegRows];
-            if (seg) cur.prefetch(rows);
-            load_segment(pol, slot, seg);
-            if (seg) cur.commit(rows);
-            decode_segment<HAS_ESC>(cur, lut, pol, slot, seg, ns);
-        }
+    cur.prime();
+    cur.start();
+    for (int seg = 0; seg < ns; seg += kSegSteps) {
+        typename Policy::Slot slot[kSegSteps];
+        uint32_t rows[kSegRows];
+        if (seg) cur.prefetch(rows);
+        load_segment(pol, slot, seg);
+        if (seg) cur.commit(rows);
+        decode_segment<HAS_ESC>(cur, lut, pol, slot, seg, ns);
     }
 }
 
@@ -243,7 +224,10 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
 // P = min(split_k*nc, NW) wavefronts of the same block (a wavefront loops when there
 // are more tasks than that), so the sum over splits and chunks never leaves the block.
 // register budget: at least this many wavefronts per SIMD must stay resident
-constexpr int min_waves(int bs) { return bs <= 1 ? 6 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
+#ifndef BHI_MIN_WAVES1
+#define BHI_MIN_WAVES1 6
+#endif
+constexpr int min_waves(int bs) { return bs <= 1 ? BHI_MIN_WAVES1 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
 
 template <class Codec, int BS, int NW>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
