@@ -85,20 +85,21 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
     return s;
 }
 
-// A task is processed in segments of kSegSteps steps; the global loads of a segment
-// (all unconditional, with clamped indices) are issued back to back before it is decoded.
-// VMEM loads complete in issue order, so a load issued on demand inside a segment would
-// make its wait drain the whole queue.
+// A task is processed in segments of kSegSteps steps; the global loads of a segment (all
+// unconditional) are issued back to back before it is decoded.  VMEM loads complete in
+// issue order, so a load issued on demand inside a segment would make its wait drain the
+// whole queue.
 //
 // Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each,
 // the ring is aligned to its 4 KB size so that a slot address is an AND and an OR).
 // Row r lives in slot r % kRingRows.  Lanes sit at different rows, yet row r of lane l
 // is always in bank l % 32: window reads are conflict free.  Every segment prefetches
-// the next kSegRows rows and commits them to the ring before it is decoded; a lane whose window is not staged (a cheap per-step
-// test) reads it from global memory instead.
+// the next kSegRows rows and commits them to the ring before it is decoded if the
+// slowest lane has made room; a lane whose window is not staged (a cheap per-step test)
+// reads it from global memory instead.
 #ifndef BHI_SEG_STEPS
-#define BHI_SEG_STEPS 8
-#define BHI_SEG_ROWS 8
+#define BHI_SEG_STEPS 4
+#define BHI_SEG_ROWS 4
 #endif
 constexpr int kSegSteps = BHI_SEG_STEPS;
 #ifndef BHI_RING_ROWS
@@ -108,18 +109,29 @@ constexpr int kRingRows = BHI_RING_ROWS;
 constexpr int kSegRows = BHI_SEG_ROWS;          // rows prefetched per segment
 constexpr int kRingSlots = kRingRows;
 constexpr int kRingWords = kRingSlots * kLanes;
+static_assert(kRingRows % kSegRows == 0 && (kRingRows & (kRingRows - 1)) == 0, "rows are committed in aligned groups");
 
 // LDS pointers are kept in their own address space: a pointer that may be LDS or global
 // turns every access into a flat load, which waits on the global-memory counter.
 typedef __attribute__((address_space(3))) uint32_t lds_u32;
 
+// Minimum over the wavefront, on the cross-lane data path (no LDS traffic): shifts within
+// rows of 16 lanes leave each row's minimum in its lane 15, two row broadcasts carry it
+// on to lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_min(uint32_t v) {
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xF, false);
+    return o < v ? o : v;
+}
+
 __device__ __forceinline__ uint32_t wave_min(uint32_t v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        uint32_t u = (uint32_t)__shfl_xor((int)v, o);
-        v = u < v ? u : v;
-    }
-    return v;
+    v = dpp_min<0x111, 0xF>(v);      // row_shr:1
+    v = dpp_min<0x112, 0xF>(v);      // row_shr:2
+    v = dpp_min<0x114, 0xF>(v);      // row_shr:4
+    v = dpp_min<0x118, 0xF>(v);      // row_shr:8
+    v = dpp_min<0x142, 0xA>(v);      // row_bcast:15 into rows 1 and 3
+    v = dpp_min<0x143, 0xC>(v);      // row_bcast:31 into rows 2 and 3
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
 // A lane's view of its task block: a bit position in its own column of rows, and the
@@ -148,9 +160,9 @@ struct RowRing {
         return (const lds_u32*)(uintptr_t)(off | (uint32_t)(uintptr_t)ring);
     }
 
-    // Stage the first rows of the block (once per task; the loads are waited for here).
+    // Stage the first kRingRows rows of the block (once per task; the loads are waited for
+    // here).  Rows past the end of a short block are filler nobody decodes.
     __device__ __forceinline__ void prime() {
-        const uint32_t hi = nrows < (uint32_t)kRingRows ? nrows : (uint32_t)kRingRows;
         uint32_t v[kRingRows];
 #pragma unroll
         for (int j = 0; j < kRingRows; ++j) {
@@ -159,40 +171,39 @@ struct RowRing {
         }
 #pragma unroll
         for (int j = 0; j < kRingRows; ++j) ring[j * kLanes] = v[j];
-        rhi = hi;
+        rhi = kRingRows;
         set_lim();
     }
 
     // windows read rows m..m+2; once the whole block is staged nothing can be missing
     __device__ __forceinline__ void set_lim() {
-        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi >= 2 ? (rhi - 2) << 5 : 0u);
+        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi - 2) << 5;
     }
 
-    // The next kSegRows rows after the staged ones, unconditionally (clamped).
+    // Can the next kSegRows rows be staged now?  Row r may replace row r - kRingRows once
+    // no window needs it, i.e. once the slowest lane is past it.  Rows are staged in whole
+    // groups: rhi stays a multiple of kSegRows and a group never wraps around the ring.
+    // Decided before the loads are issued so that they need not be issued in vain (and so
+    // that the compiler cannot sink them behind the decision, next to their use).
+    __device__ __forceinline__ bool room() const {
+        const uint32_t mmin = uniform(wave_min(pos)) >> 5;
+        return rhi < nrows && rhi + kSegRows <= mmin + kRingRows;
+    }
+
+    // The next kSegRows rows after the staged ones: one address, immediate offsets.  Rows
+    // past the end of the block belong to the next block or to the zero pad that ends the
+    // stream; they are loaded, staged, never decoded.
     __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) const {
+        const uint32_t* p = bp + (size_t)rhi * kLanes;
 #pragma unroll
-        for (int j = 0; j < kSegRows; ++j) {
-            uint32_t r = rhi + j;
-            r = r < nrows ? r : nrows - 1;
-            v[j] = bp[(size_t)r * kLanes];
-        }
+        for (int j = 0; j < kSegRows; ++j) v[j] = p[j * kLanes];
     }
 
-    // Move the prefetched rows into the ring as far as the slowest lane allows (row r may
-    // replace row r - kRingRows once no window needs it).
     __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
-        const uint32_t mmin = uniform(wave_min(pos) >> 5);
-        uint32_t hi = mmin + kRingRows;
-        hi = hi < nrows ? hi : nrows;
-        hi = hi < rhi + kSegRows ? hi : rhi + kSegRows;
+        lds_u32* dst = ring + (rhi & (kRingRows - 1)) * kLanes;
 #pragma unroll
-        for (int j = 0; j < kSegRows; ++j) {
-            if (rhi + j < hi) {
-                const uint32_t slot = (rhi + j) & (kRingRows - 1);
-                ring[slot * kLanes] = v[j];
-            }
-        }
-        rhi = hi > rhi ? hi : rhi;
+        for (int j = 0; j < kSegRows; ++j) dst[j * kLanes] = v[j];
+        rhi += kSegRows;
         set_lim();
     }
 
@@ -222,6 +233,20 @@ struct RowRing {
     }
 };
 
+// The table entry selected by bits 2..13 of a (pre-shifted) window.
+#if defined(BHI_PROBE_SWZ)
+__device__ __forceinline__ uint32_t table_swizzle(uint32_t a) { return a ^ ((a >> 5) & 0x7Cu); }
+#else
+__device__ __forceinline__ uint32_t table_swizzle(uint32_t a) { return a; }
+#endif
+__device__ __forceinline__ uint32_t table_entry(const char* tb, uint32_t w) {
+    const uint32_t a = table_swizzle(w & kTableMask);
+#if defined(BHI_PROBE_DUP)
+    (void)*(const volatile uint32_t*)(tb + (a ^ 0x1000u));
+#endif
+    return *(const uint32_t*)(tb + a);
+}
+
 // Per-lane Huffman bit cursor.  pos = bit position - 2: the window is kept shifted left
 // by two so that `window & 0x3FFC` is the byte address of the table entry.
 struct HuffCursor : RowRing {
@@ -244,16 +269,16 @@ struct HuffCursor : RowRing {
         const char* tb = (const char*)table;
         const uint32_t c = pos & 31u;
         const uint32_t wlo = __builtin_amdgcn_alignbit(hi, lo, c);
-        e[0] = *(const uint32_t*)(tb + (wlo & kTableMask));
+        e[0] = table_entry(tb, wlo);
         const uint32_t w1 = wlo >> (e[0] & 31u);
-        e[1] = *(const uint32_t*)(tb + (w1 & kTableMask));
+        e[1] = table_entry(tb, w1);
         const uint32_t whi = __builtin_amdgcn_alignbit(nx, hi, c);
         if (HAS_ESC) {
             const uint32_t s01 = (e[0] & kLenMask) + (e[1] & kLenMask);
             const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, s01);
-            e[2] = *(const uint32_t*)(tb + (w2 & kTableMask));
+            e[2] = table_entry(tb, w2);
             const uint32_t w3 = w2 >> (e[2] & 31u);
-            e[3] = *(const uint32_t*)(tb + (w3 & kTableMask));
+            e[3] = table_entry(tb, w3);
             const uint32_t sum = s01 + (e[2] & kLenMask) + (e[3] & kLenMask);
             pos += sum & 0x3Fu;
             if (__builtin_expect(ballot(sum >= kEscStep) != 0, 0)) escapes(e);
@@ -262,9 +287,9 @@ struct HuffCursor : RowRing {
             // sum of raw entries are the sum of the lengths (at most 48)
             const uint32_t t01 = e[0] + e[1];
             const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, t01);
-            e[2] = *(const uint32_t*)(tb + (w2 & kTableMask));
+            e[2] = table_entry(tb, w2);
             const uint32_t w3 = w2 >> (e[2] & 31u);
-            e[3] = *(const uint32_t*)(tb + (w3 & kTableMask));
+            e[3] = table_entry(tb, w3);
             pos += (t01 + e[2] + e[3]) & 0x3Fu;
         }
     }

@@ -17,7 +17,11 @@ template <int WORDS>
 __device__ __forceinline__ void load_table(uint32_t* __restrict__ lds, const uint32_t* __restrict__ g) {
     const uint4* src = (const uint4*)g;
     uint4* dst = (uint4*)lds;
+#if defined(BHI_PROBE_SWZ)
+    for (int i = threadIdx.x; i < WORDS; i += blockDim.x) *(uint32_t*)((char*)lds + table_swizzle(4u * i)) = g[i];
+#else
     for (int i = threadIdx.x; i < WORDS / 4; i += blockDim.x) dst[i] = src[i];
+#endif
 }
 
 struct Shape {
@@ -32,18 +36,12 @@ struct Shape {
 // compute phase; `use(...)` receives the lane's four rebuilt BF16 pairs (columns 0..7 of
 // its row in step t).  Because every load is unconditional the compiler can count the
 // outstanding ones and make each step wait for exactly its own operands.
-template <class Policy>
-__device__ __forceinline__ void load_segment(const Policy& pol, typename Policy::Slot (&slot)[kSegSteps], int t0) {
-#pragma unroll
-    for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], t0 + i);
-}
-
-template <bool HAS_ESC, class Cursor, class Policy>
+template <bool FULL, bool HAS_ESC, class Cursor, class Policy>
 __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut, Policy& pol,
                                                const typename Policy::Slot (&slot)[kSegSteps], int t0, int ns) {
 #pragma unroll
     for (int i = 0; i < kSegSteps; ++i) {
-        if (t0 + i < ns) {
+        if (FULL || t0 + i < ns) {
             const typename Policy::Piped piped = pol.take(slot[i], i, t0 + i);
             uint32_t e[4];
             cur.template step<HAS_ESC>(lut, e);
@@ -58,18 +56,30 @@ __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut,
     }
 }
 
+// Whole segments load their operands from one address with immediate offsets and decode
+// without per-step guards; a last, shorter segment clamps its step indices instead.
 template <bool HAS_ESC, class Cursor, class Policy>
 __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns) {
     pol.prime();
     cur.prime();
     cur.start();
-    for (int seg = 0; seg < ns; seg += kSegSteps) {
-        typename Policy::Slot slot[kSegSteps];
-        uint32_t rows[kSegRows];
-        if (seg) cur.prefetch(rows);
-        load_segment(pol, slot, seg);
-        if (seg) cur.commit(rows);
-        decode_segment<HAS_ESC>(cur, lut, pol, slot, seg, ns);
+    typename Policy::Slot slot[kSegSteps];
+    uint32_t rows[kSegRows];
+    int seg = 0;
+    for (; seg + kSegSteps <= ns; seg += kSegSteps) {
+        const bool stage = cur.room();
+        if (stage) cur.prefetch(rows);
+        pol.load_full(slot, seg);
+        if (stage) cur.commit(rows);
+        decode_segment<true, HAS_ESC>(cur, lut, pol, slot, seg, ns);
+    }
+    if (seg < ns) {
+        const bool stage = cur.room();
+        if (stage) cur.prefetch(rows);
+#pragma unroll
+        for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], seg + i);
+        if (stage) cur.commit(rows);
+        decode_segment<false, HAS_ESC>(cur, lut, pol, slot, seg, ns);
     }
 }
 
@@ -91,6 +101,11 @@ struct StorePolicy {
     __device__ __forceinline__ void load(Slot& s, int t) const {
         t = t < last ? t : last;
         s.rem = rem0[(size_t)t * kLanes];
+    }
+    __device__ __forceinline__ void load_full(Slot (&s)[kSegSteps], int t0) const {
+        const uint2* p = rem0 + (size_t)t0 * kLanes;
+#pragma unroll
+        for (int i = 0; i < kSegSteps; ++i) s[i].rem = p[i * kLanes];
     }
     __device__ __forceinline__ Piped take(const Slot&, int, int) const { return Piped{}; }
     __device__ __forceinline__ void use(const Piped&, int t, const uint32_t (&w)[4]) const {
@@ -149,6 +164,17 @@ struct MfmaPolicy {
         s.rem = rem0[(size_t)t * kLanes];
         if (QUARTER) s.x.x = xq0[(size_t)t * (kStepCols / 2)];
         else if (!PIPED) s.x = x0[0][(size_t)t * (kStepCols / 8)];
+    }
+    __device__ __forceinline__ void load_full(Slot (&s)[kSegSteps], int t0) const {
+        const uint2* pr = rem0 + (size_t)t0 * kLanes;
+        const uint32_t* pq = xq0 + (size_t)t0 * (kStepCols / 2);
+        const uint4* px = x0[0] + (size_t)t0 * (kStepCols / 8);
+#pragma unroll
+        for (int i = 0; i < kSegSteps; ++i) {
+            s[i].rem = pr[i * kLanes];
+            if (QUARTER) s[i].x.x = pq[i * (kStepCols / 2)];
+            else if (!PIPED) s[i].x = px[i * (kStepCols / 8)];
+        }
     }
     __device__ __forceinline__ Piped take(const Slot& s, int i, int t) {
         Piped p;
