@@ -25,6 +25,7 @@ HBM_PEAK_GBS = 8000.0
 LAYERS = [("qkv_proj", 4608, 3584), ("o_proj", 3584, 3584), ("gate_proj", 18944, 3584),
           ("up_proj", 18944, 3584), ("down_proj", 3584, 18944)]
 COPIES = 2
+ROTATE_BYTES = 640 << 20
 STD = 0.02
 # HBM bytes per launch of the dominant kernel (18944x3584), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, each scaled by the same counter's reading for the 256 MiB
@@ -169,23 +170,31 @@ def main():
     sec = time_launches(step, args.steps, args.warmup, launches_per_graph=COPIES)
     gbs = block_bytes / sec / 1e9
 
-    # per-layer timing and the roofline of the dominant kernel
+    # Per-layer timing and the roofline of the dominant kernel.  A layer alone must not be
+    # served by the 256 MB last-level cache either: it rotates over clones of its module
+    # (same bytes at different addresses) that add up to at least ROTATE_BYTES.
+    import copy
+
+    def rotating(mod):
+        n = max(2, -(-ROTATE_BYTES // weight_bytes(mod)))
+        return [mod] + [copy.deepcopy(mod) for _ in range(n - 1)]
+
     per_layer = {}
+    t_dom = None
     for li, (name, M, K) in enumerate(LAYERS):
+        if li == 3:                               # up_proj is gate_proj's twin: same shape, same kernel
+            per_layer[name] = per_layer["gate_proj"]
+            continue
+        mods = rotating(blocks[0][li])
         st = {"i": 0}
 
-        def one(li=li, st=st):
-            F.linear(xs[li], blocks[st["i"] % COPIES][li])
+        def one(li=li, st=st, mods=mods):
+            F.linear(xs[li], mods[st["i"] % len(mods)])
             st["i"] += 1
-        per_layer[name] = time_launches(one, max(50, args.steps), args.warmup, launches_per_graph=COPIES)
-    big = [2, 3]                                  # gate and up of both copies: four distinct 96 MB streams
-    st = {"i": 0}
-
-    def dominant():
-        i = st["i"]
-        F.linear(xs[big[i % 2]], blocks[(i // 2) % COPIES][big[i % 2]])
-        st["i"] += 1
-    t_dom = time_launches(dominant, max(100, args.steps), args.warmup, launches_per_graph=2 * COPIES)
+        per_layer[name] = time_launches(one, max(100, args.steps), args.warmup, launches_per_graph=len(mods))
+        if li == 2:
+            t_dom = per_layer[name]
+        del mods
     dom_bytes = gemv_bytes(blocks[0][2], bs, LAYERS[2][1], LAYERS[2][2])
     achieved = dom_bytes / t_dom / 1e9
 

@@ -56,10 +56,11 @@ __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_bal
 
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
-// Table entry: len in bits 4..0, ESC flag in bit 15, exponent a in bits 14..7 and
-// exponent b in bits 30..23 -- where a packed pair of BF16 values keeps them.
-constexpr uint32_t kLenMask = 0x801Fu;       // length and ESC flag
-constexpr uint32_t kEscStep = 0x8000u;       // what an ESC entry adds to the cursor
+// Table entry: len in bits 4..0 (bits 5, 6 clear), exponent a in bits 14..7 and exponent
+// b in bits 30..23 -- where a packed pair of BF16 values keeps them -- and the ESC flag in
+// bit 31.  The low six bits of a sum of raw entries are therefore the sum of their
+// lengths (at most 48), and an OR of entries is negative iff one of them is an ESC.
+constexpr uint32_t kEscFlag = 0x80000000u;
 
 // Two BF16 values from (table entry, rem bytes).  `z` holds [rb, rb, ra, ra]: the sign
 // comes from the upper copy of each rem byte, the mantissa from the lower copy.
@@ -90,10 +91,11 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
 // issue order, so a load issued on demand inside a segment would make its wait drain the
 // whole queue.
 //
-// Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each,
-// the ring is aligned to its 4 KB size so that a slot address is an AND and an OR).
-// Row r lives in slot r % kRingRows.  Lanes sit at different rows, yet row r of lane l
-// is always in bank l % 32: window reads are conflict free.  Every segment prefetches
+// Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each).
+// Row r lives in slot r % kRingRows; slots 0 and 1 are mirrored behind the last slot so
+// that the three rows of a window are always at +0, +256 and +512 bytes of one address.
+// Lanes sit at different rows, yet row r of lane l is always in bank l % 32: window reads
+// are conflict free.  Every segment prefetches
 // the next kSegRows rows and commits them to the ring before it is decoded if the
 // slowest lane has made room; a lane whose window is not staged (a cheap per-step test)
 // reads it from global memory instead.
@@ -107,9 +109,10 @@ constexpr int kSegSteps = BHI_SEG_STEPS;
 #endif
 constexpr int kRingRows = BHI_RING_ROWS;
 constexpr int kSegRows = BHI_SEG_ROWS;          // rows prefetched per segment
-constexpr int kRingSlots = kRingRows;
+constexpr int kRingSlots = kRingRows + 2;   // slots 0 and 1 are mirrored behind the last one
 constexpr int kRingWords = kRingSlots * kLanes;
-static_assert(kRingRows % kSegRows == 0 && (kRingRows & (kRingRows - 1)) == 0, "rows are committed in aligned groups");
+static_assert(kRingRows % kSegRows == 0 && (kRingRows & (kRingRows - 1)) == 0 && kSegRows >= 2,
+              "rows are committed in aligned groups; the group at slot 0 carries both mirrored rows");
 
 // LDS pointers are kept in their own address space: a pointer that may be LDS or global
 // turns every access into a flat load, which waits on the global-memory counter.
@@ -153,11 +156,9 @@ struct RowRing {
         lim = 0;
     }
 
-    // LDS address of this lane's word of row (p >> 5) + k: the ring base has its bits
-    // 8..11 clear, the row index lands there.
-    __device__ __forceinline__ const lds_u32* slot_of(uint32_t p, int k) const {
-        const uint32_t off = ((p << 3) + 256u * k) & ((kRingRows - 1) * 256u);
-        return (const lds_u32*)(uintptr_t)(off | (uint32_t)(uintptr_t)ring);
+    // This lane's word of row p >> 5; the next two rows follow at +kLanes, +2*kLanes words.
+    __device__ __forceinline__ const lds_u32* slot_of(uint32_t p) const {
+        return ring + ((p >> 5) & (kRingRows - 1)) * kLanes;
     }
 
     // Stage the first kRingRows rows of the block (once per task; the loads are waited for
@@ -171,6 +172,8 @@ struct RowRing {
         }
 #pragma unroll
         for (int j = 0; j < kRingRows; ++j) ring[j * kLanes] = v[j];
+        ring[kRingRows * kLanes] = v[0];
+        ring[(kRingRows + 1) * kLanes] = v[1];
         rhi = kRingRows;
         set_lim();
     }
@@ -203,6 +206,10 @@ struct RowRing {
         lds_u32* dst = ring + (rhi & (kRingRows - 1)) * kLanes;
 #pragma unroll
         for (int j = 0; j < kSegRows; ++j) dst[j * kLanes] = v[j];
+        if ((rhi & (kRingRows - 1)) == 0) {
+            ring[kRingRows * kLanes] = v[0];
+            ring[(kRingRows + 1) * kLanes] = v[1];
+        }
         rhi += kSegRows;
         set_lim();
     }
@@ -212,9 +219,10 @@ struct RowRing {
         if (__builtin_expect(ballot(pos >= lim) != 0, 0)) {
             fetch_slow(lo, hi, nx);
         } else {
-            lo = *slot_of(pos, 0);
-            hi = *slot_of(pos, 1);
-            nx = *slot_of(pos, 2);
+            const lds_u32* w = slot_of(pos);
+            lo = w[0];
+            hi = w[kLanes];
+            nx = w[2 * kLanes];
         }
     }
 
@@ -224,7 +232,8 @@ struct RowRing {
         const uint32_t m = pos >> 5;
         const bool staged = pos < lim;
         // both reads are always in range (the stream ends in a zero pad), then pick per lane
-        const uint32_t l0 = *slot_of(pos, 0), l1 = *slot_of(pos, 1), l2 = *slot_of(pos, 2);
+        const lds_u32* w = slot_of(pos);
+        const uint32_t l0 = w[0], l1 = w[kLanes], l2 = w[2 * kLanes];
         const uint32_t* g = bp + (size_t)(staged ? 0u : m) * kLanes;
         const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
         lo = staged ? l0 : g0;
@@ -273,24 +282,15 @@ struct HuffCursor : RowRing {
         const uint32_t w1 = wlo >> (e[0] & 31u);
         e[1] = table_entry(tb, w1);
         const uint32_t whi = __builtin_amdgcn_alignbit(nx, hi, c);
+        const uint32_t t01 = e[0] + e[1];
+        const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, t01);
+        e[2] = table_entry(tb, w2);
+        const uint32_t w3 = w2 >> (e[2] & 31u);
+        e[3] = table_entry(tb, w3);
+        pos += (t01 + e[2] + e[3]) & 0x3Fu;
         if (HAS_ESC) {
-            const uint32_t s01 = (e[0] & kLenMask) + (e[1] & kLenMask);
-            const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, s01);
-            e[2] = table_entry(tb, w2);
-            const uint32_t w3 = w2 >> (e[2] & 31u);
-            e[3] = table_entry(tb, w3);
-            const uint32_t sum = s01 + (e[2] & kLenMask) + (e[3] & kLenMask);
-            pos += sum & 0x3Fu;
-            if (__builtin_expect(ballot(sum >= kEscStep) != 0, 0)) escapes(e);
-        } else {
-            // lengths sit in bits 4..0 and bits 5, 6 are clear, so the low six bits of a
-            // sum of raw entries are the sum of the lengths (at most 48)
-            const uint32_t t01 = e[0] + e[1];
-            const uint32_t w2 = __builtin_amdgcn_alignbit(whi, wlo, t01);
-            e[2] = table_entry(tb, w2);
-            const uint32_t w3 = w2 >> (e[2] & 31u);
-            e[3] = table_entry(tb, w3);
-            pos += (t01 + e[2] + e[3]) & 0x3Fu;
+            const uint32_t any = e[0] | e[1] | e[2] | e[3];
+            if (__builtin_expect(ballot((int32_t)any < 0) != 0, 0)) escapes(e);
         }
     }
 
@@ -298,7 +298,7 @@ struct HuffCursor : RowRing {
     __device__ __forceinline__ void escapes(uint32_t (&e)[4]) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            bool esc = (e[q] & kEscStep) != 0;
+            bool esc = (int32_t)e[q] < 0;
             uint64_t m = ballot(esc);
             if (esc) {
                 uint32_t v = *(ep - 1 - (eptr + lane_rank(m)));

@@ -219,7 +219,7 @@ __global__ __launch_bounds__(NW * kLanes)
 void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
                            uint16_t* __restrict__ Y, const uint32_t* __restrict__ offsets,
                            const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
-    __shared__ __align__(4096) uint32_t rings[NW][kRingWords];
+    __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
     load_table<Codec::kTableWords>(lut, table);
     __syncthreads();
@@ -262,7 +262,7 @@ void gemv_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__
                          const uint32_t* __restrict__ offsets, const uint32_t* __restrict__ table,
                          const uint8_t* __restrict__ header, Shape s, int P, int groups_per_block) {
     // The partial sums reuse the rings once every task of the block is done.
-    __shared__ __align__(4096) uint32_t rings[NW][kRingWords];
+    __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
     load_table<Codec::kTableWords>(lut, table);
     __syncthreads();

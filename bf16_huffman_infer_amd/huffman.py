@@ -19,7 +19,7 @@ import numpy as np
 import torch
 
 TABLE_BITS = 12
-ESC_FLAG = 1 << 15
+ESC_FLAG = 1 << 31
 ESC_INDEX = 65536
 ESC_SIDE_BITS = 32            # one stream word per escaped pair
 MAX_CODED = 3072              # never give more than this many pairs a code of their own
@@ -74,7 +74,7 @@ class LUTHuffmanEncoder:
 
     * ``enc_table``  uint32 ``[65537]``: ``code | len<<16`` per pair (0 = escaped), ESC in
       slot 65536; code bits are emitted LSB first.
-    * ``dec_table``  uint32 ``[4096]``: ``len | a<<7 | b<<23`` (``| 1<<15`` for ESC): the two
+    * ``dec_table``  uint32 ``[4096]``: ``len | a<<7 | b<<23`` (``| 1<<31`` for ESC): the two
       exponents already sit at their BF16 bit positions of a packed pair.
     * ``LUT1``       the decode table viewed as uint8 ``[16384]`` -- the module buffer.
     * ``LUT2..LUT4`` uint8 ``[256]`` filled with 255: the reference's deeper cascade

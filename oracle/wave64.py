@@ -20,7 +20,7 @@ code        one length-limited (<= 12 bit) Huffman code over exponent *pairs*
             ``a | b<<8`` (a = even column) plus an ESC word; code bits are consumed
             LSB first.  ``dec`` is the 4096-entry decode table indexed by the next 12
             stream bits: ``len | a<<7 | b<<23`` (the exponents sit where a packed BF16
-            pair needs them); ESC entries are ``len | 1<<15``.  The two raw exponents
+            pair needs them); ESC entries are ``len | 1<<31``.  The two raw exponents
             of an escaped pair are not in the bitstream: they sit in the task's
             escape list.
 lane bits   a lane's codes are concatenated from bit 2 of its private bitstring (the
@@ -54,7 +54,7 @@ PAIRS_PER_STEP = 4
 WINDOW_WORDS = 3           # words of its bitstring a lane looks at per step
 HEADER_BITS = 2            # dummy bits in front of every lane's codes
 TABLE_BITS = 12
-ESC_FLAG = 1 << 15
+ESC_FLAG = 1 << 31
 TARGET_TASKS = 6144        # wavefronts one MI355X keeps resident: 256 CUs x 4 SIMDs x 6
 MIN_CHUNK_STEPS = 4
 MAX_CHUNKS = 4
@@ -210,7 +210,7 @@ def _decode_tasks(words: np.ndarray, base: np.ndarray, end: np.ndarray, ns: int,
         for q in range(PAIRS_PER_STEP):
             e = dec64[((win >> U(HEADER_BITS)) & U((1 << TABLE_BITS) - 1)).astype(np.int64)]
             ln = (e & U(0x1F)).astype(np.int64)
-            esc = ((e >> U(15)) & U(1)).astype(bool)
+            esc = ((e >> U(31)) & U(1)).astype(bool)
             a = ((e >> U(7)) & U(0xFF)).astype(np.uint8)
             b = ((e >> U(23)) & U(0xFF)).astype(np.uint8)
             if esc.any():
