@@ -211,7 +211,7 @@ def main():
             sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),
         "block_steps_per_s": round(1.0 / sec, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
-        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{'HuffCodec' if args.algo == 'huffman' else 'AnsCodec'}, {bs}, 8> "
+        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{'HuffCodec' if args.algo == 'huffman' else 'AnsCodec'}, {bs}, 4> "
                                f"18944x3584",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),

@@ -22,7 +22,7 @@ constexpr int kStepCols = 128;
 constexpr int kPairsPerStep = 4;
 constexpr int kWindowWords = 3;
 constexpr int kHeaderBits = 2;
-constexpr int kTableBits = 12;
+constexpr int kTableBits = 11;
 constexpr int kTableEntries = 1 << kTableBits;
 constexpr uint32_t kTableMask = (kTableEntries - 1) << 2;   // byte address mask
 constexpr int kMaxBatch = 8;
@@ -36,7 +36,7 @@ constexpr int kTargetTasks = BHI_TARGET_TASKS;      // wavefronts kept resident:
 constexpr int kMinChunkSteps = 4;
 constexpr int kMaxChunks = 4;
 constexpr int kMaxTaskSteps = 128;
-constexpr int kWavesPerBlock = 8;
+constexpr int kWavesPerBlock = 4;
 constexpr int kBlockThreads = kWavesPerBlock * kLanes;
 
 __host__ __device__ inline int chunks_per_group(int M, int Ks, int split_k) {
@@ -257,7 +257,7 @@ __device__ __forceinline__ uint32_t table_entry(const char* tb, uint32_t w) {
 }
 
 // Per-lane Huffman bit cursor.  pos = bit position - 2: the window is kept shifted left
-// by two so that `window & 0x3FFC` is the byte address of the table entry.
+// by two so that `window & kTableMask` is the byte address of the table entry.
 struct HuffCursor : RowRing {
     uint32_t eptr;           // wave-uniform: escape entries consumed so far
     const uint32_t* ep;      // one past the task block (escape list grows down from here)

@@ -69,7 +69,7 @@ void huffman_encode_kernel(const uint8_t* __restrict__ data, const uint32_t* __r
                 out[total - 1 - (eptr + lane_rank(m))] = pr[q];
             }
             eptr += (uint32_t)__builtin_popcountll(m);
-            acc |= (uint64_t)(en & 0xFFFFu) << fill;          // fill < 32, code <= 12 bits
+            acc |= (uint64_t)(en & 0xFFFFu) << fill;          // fill < 32, code <= 11 bits
             fill += en >> 16;
             if (fill >= 32u) {
                 out[(size_t)row * kLanes + lane] = (uint32_t)acc;
@@ -97,7 +97,7 @@ extern "C" int bhi_huffman_decode(const void* A_rem, const void* A_exp, int64_t 
     if (!A_rem || !A_exp || !Y || !offsets || !LUT1 || !code_lengths) return bhi_fail(BHI_EINVAL, "null pointer");
     Shape s;
     if (lut1_bytes != (int64_t)kTableEntries * 4)
-        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 4096 four-byte pair entries");
+        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 2048 four-byte pair entries");
     if (int rc = check_shape(split_k, M, Ks, exp_words, &s)) return rc;
     launch_decode<HuffCodec>(A_rem, A_exp, Y, offsets, LUT1, code_lengths, s, (hipStream_t)stream);
     return bhi_launch_status("huffman_decode");
@@ -113,7 +113,7 @@ extern "C" int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64
     if (batch > kMaxBatch) return bhi_fail(BHI_EBATCH, "fused GEMV supports batch <= 8");
     Shape s;
     if (lut1_bytes != (int64_t)kTableEntries * 4)
-        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 4096 four-byte pair entries");
+        return bhi_fail(BHI_ELAYOUT, "LUT1 must hold 2048 four-byte pair entries");
     if (int rc = check_shape(split_k, M, Ks, exp_words, &s)) return rc;
     launch_gemv_batch<HuffCodec>(batch, A_rem, A_exp, X, Y, offsets, LUT1, code_lengths, s, (hipStream_t)stream);
     return bhi_launch_status("gemv_bf16_huffman");
@@ -121,7 +121,7 @@ extern "C" int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64
 
 extern "C" int64_t bhi_encode_capacity(int n_steps) {
     if (n_steps < 1) return 0;
-    // every lane full of 12-bit codes + every pair escaped + alignment
+    // every lane full of longest codes + every pair escaped + alignment
     int64_t lane_words = ((int64_t)kHeaderBits + (int64_t)n_steps * kPairsPerStep * kTableBits + 31) / 32;
     return (int64_t)kLanes * lane_words + (int64_t)n_steps * kPairsPerStep * kLanes + kAlignWords;
 }

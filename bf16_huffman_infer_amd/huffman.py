@@ -3,26 +3,26 @@
 Counterpart of the reference's ``LUTHuffmanEncoder.build_lut``
 (``bf16_huffman_infer/huffman.py:347-361``), redesigned for a 64-lane decoder: the
 coded alphabet is the set of exponent *pairs* ``a | b<<8`` (two horizontally adjacent
-weights), every code is at most 12 bits long, and one 4096-entry table resolves the
-next 12 stream bits to both exponents at once.  The reference instead limits single
+weights), every code is at most 11 bits long, and one 2048-entry table resolves the
+next 11 stream bits to both exponents at once.  The reference instead limits single
 symbol codes to 32 bits and perturbs the frequencies until the codes fit four
 256-entry byte tables (``huffman.py:84-218``); that cascade costs two dependent
 shared-memory reads per exponent, here one read yields two exponents.
 
 Pairs that are too rare to deserve a code share one ESC code; their two raw bytes
 travel in a side list of the stream, so the in-band cost of any pair is bounded by
-12 bits and the decoder's bit window never overflows.
+11 bits and the decoder's bit window never overflows.
 """
 from typing import Dict, Tuple, Union
 
 import numpy as np
 import torch
 
-TABLE_BITS = 12
+TABLE_BITS = 11
 ESC_FLAG = 1 << 31
 ESC_INDEX = 65536
 ESC_SIDE_BITS = 32            # one stream word per escaped pair
-MAX_CODED = 3072              # never give more than this many pairs a code of their own
+MAX_CODED = 1536              # never give more than this many pairs a code of their own
 
 
 def package_merge(weights, max_len: int):
@@ -68,15 +68,15 @@ def _bit_reverse(v: int, n: int) -> int:
 
 
 class LUTHuffmanEncoder:
-    """Pair-alphabet, 12-bit-limited canonical Huffman code with its two tables.
+    """Pair-alphabet, 11-bit-limited canonical Huffman code with its two tables.
 
     After :meth:`build_lut`:
 
     * ``enc_table``  uint32 ``[65537]``: ``code | len<<16`` per pair (0 = escaped), ESC in
       slot 65536; code bits are emitted LSB first.
-    * ``dec_table``  uint32 ``[4096]``: ``len | a<<7 | b<<23`` (``| 1<<31`` for ESC): the two
+    * ``dec_table``  uint32 ``[2048]``: ``len | a<<7 | b<<23`` (``| 1<<31`` for ESC): the two
       exponents already sit at their BF16 bit positions of a packed pair.
-    * ``LUT1``       the decode table viewed as uint8 ``[16384]`` -- the module buffer.
+    * ``LUT1``       the decode table viewed as uint8 ``[8192]`` -- the module buffer.
     * ``LUT2..LUT4`` uint8 ``[256]`` filled with 255: the reference's deeper cascade
       levels have no job when no code is longer than the first-level window.
     * ``code_lengths`` uint8 ``[256]``: a format header (version, table bits, ESC length,

@@ -16,15 +16,15 @@ step        128 columns x 4 rows.  Lane ``l = 4*b + i`` owns row ``4g+i`` and th
             columns ``128*t + 8*b + j`` (j = 0..7): 4 exponent *pairs* per step.
 rem plane   uint8 ``[split_k, M, Ks]``; the ``4*Ks`` bytes of (k, g) hold step ``t``,
             lane ``l``, column ``j`` at byte ``512*t + 8*l + j``.
-code        one length-limited (<= 12 bit) Huffman code over exponent *pairs*
+code        one length-limited (<= 11 bit) Huffman code over exponent *pairs*
             ``a | b<<8`` (a = even column) plus an ESC word; code bits are consumed
-            LSB first.  ``dec`` is the 4096-entry decode table indexed by the next 12
+            LSB first.  ``dec`` is the 2048-entry decode table indexed by the next 11
             stream bits: ``len | a<<7 | b<<23`` (the exponents sit where a packed BF16
             pair needs them); ESC entries are ``len | 1<<31``.  The two raw exponents
             of an escaped pair are not in the bitstream: they sit in the task's
             escape list.
 lane bits   a lane's codes are concatenated from bit 2 of its private bitstring (the
-            decoder keeps its window shifted left by two so that ``window & 0x3FFC`` is
+            decoder keeps its window shifted left by two so that ``window & 0x1FFC`` is
             the byte address of the table entry) and the bitstring is cut into
             32-bit words.
 task block  ``[W rows of 64 words][escape list][zero pad]``, a multiple of 4 words:
@@ -53,7 +53,7 @@ STEP_COLS = 128
 PAIRS_PER_STEP = 4
 WINDOW_WORDS = 3           # words of its bitstring a lane looks at per step
 HEADER_BITS = 2            # dummy bits in front of every lane's codes
-TABLE_BITS = 12
+TABLE_BITS = 11
 ESC_FLAG = 1 << 31
 TARGET_TASKS = 6144        # wavefronts one MI355X keeps resident: 256 CUs x 4 SIMDs x 6
 MIN_CHUNK_STEPS = 4
@@ -395,7 +395,7 @@ def decode_ans(rem_packed: np.ndarray, exp_words: np.ndarray, offsets: np.ndarra
 def check_tables(dec: np.ndarray, enc: np.ndarray) -> None:
     """Consistency of a decode table with its encoder table (raises AssertionError).
 
-    Every 12-bit index must resolve to exactly the pair (or ESC) whose LSB-first code
+    Every table index must resolve to exactly the pair (or ESC) whose LSB-first code
     is a prefix of the index; the code is therefore prefix-free and complete.
     """
     assert dec.shape == (1 << TABLE_BITS,) and enc.shape == (ESC_INDEX + 1,)

@@ -172,25 +172,26 @@ def test_wave64_and_reference_layout_agree():
 
 def test_wave64_escape_list_and_cursor_edges():
     """Hand-made code: three coded pairs and ESC; rows alternate so that every lane meets
-    escapes, 1-bit codes and 12-bit codes, and cursors cross words at different steps."""
+    escapes, 1-bit codes and longest codes, and cursors cross words at different steps."""
     enc = np.zeros(wave64.ESC_INDEX + 1, dtype=np.uint32)
     dec = np.zeros(1 << wave64.TABLE_BITS, dtype=np.uint32)
-    table = {0x7878: (0b0, 1), 0x7979: (0b01, 2), 0x7A7A: (0b111111111011, 12), wave64.ESC_INDEX: (0b011111111011, 12)}
+    TB = wave64.TABLE_BITS
+    table = {0x7878: (0b0, 1), 0x7979: (0b01, 2), 0x7A7A: ((1 << TB) - 5, TB), wave64.ESC_INDEX: ((1 << (TB - 1)) - 5, TB)}
     for p, (code, ln) in table.items():
         enc[p] = code | (ln << 16)
-    # complete the code with filler pairs so that every 12-bit index resolves
+    # complete the code with filler pairs so that every table index resolves
     filler = 0x0101
-    used = np.zeros(1 << 12, dtype=bool)
+    used = np.zeros(1 << TB, dtype=bool)
     for p, (code, ln) in table.items():
-        idx = code + (np.arange(1 << (12 - ln)) << ln)
+        idx = code + (np.arange(1 << (TB - ln)) << ln)
         used[idx] = True
-    # every unused index becomes its own 12-bit code of a filler pair
+    # every unused index becomes its own longest code of a filler pair
     for idx in np.nonzero(~used)[0]:
-        enc[filler] = int(idx) | (12 << 16)
-        table[filler] = (int(idx), 12)
+        enc[filler] = int(idx) | (TB << 16)
+        table[filler] = (int(idx), TB)
         filler += 1
     for p, (code, ln) in table.items():
-        idx = code + (np.arange(1 << (12 - ln)) << ln)
+        idx = code + (np.arange(1 << (TB - ln)) << ln)
         dec[idx] = (ln | wave64.ESC_FLAG) if p == wave64.ESC_INDEX else (ln | ((p & 0xFF) << 7) | ((p >> 8) << 23))
     wave64.check_tables(dec, enc)
     rng = np.random.default_rng(0)
