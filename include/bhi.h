@@ -57,7 +57,7 @@ const char* bhi_last_error_string(void);
  *   X       bf16   [batch, split_k*Ks]
  *   Y       bf16   [batch, M]        written
  *   offsets int32  [split_k, M]
- *   LUT1    uint8  [lut1_bytes]      pair decode table, lut1_bytes = 4 << table bits
+ *   LUT1    uint8  [lut1_bytes]      pair decode table, lut1_bytes = 4 << table bits (8192)
  *   LUT2..4 uint8 [256] (carried for the op signature; not read)
  *   code_lengths uint8 [256]        format header: version, table bits, ESC length, has-escapes */
 int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64_t exp_words,
