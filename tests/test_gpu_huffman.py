@@ -96,3 +96,30 @@ def test_ops_reject_cpu_tensors_and_big_batch(cuda):
     with pytest.raises(RuntimeError, match="batch"):
         ops.gemv_bf16_huffman(mod.rem, mod.exp, x, out, mod.offsets, mod.LUT1, mod.LUT2, mod.LUT3, mod.LUT4,
                               mod.code_lengths)
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("kind,M,K", [
+    ("gauss", 4096, 4096), ("gauss", 4608, 3584), ("gauss", 3584, 3584), ("gauss", 18944, 3584),
+    ("gauss", 3584, 18944), ("t3", 12288, 4096), ("t3", 4096, 12288),
+])
+def test_full_size_layers_round_trip(cuda, algo, kind, M, K):
+    """The layer shapes of the benchmark configurations at full size: the decoded weight is
+    the original bit for bit, and the fused GEMV agrees with a matmul on that weight."""
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight
+    g = torch.Generator(device="cuda").manual_seed(M + K)
+    if kind == "gauss":
+        w = (torch.randn(M, K, generator=g, device="cuda") * 0.02).bfloat16()
+    else:
+        torch.manual_seed(M + K)
+        w = (torch.distributions.StudentT(3.0).sample((M, K)) * (0.02 / 3 ** 0.5)).bfloat16().cuda()
+    mod = (HuffmanWeight if algo == "huffman" else ANSWeight).compress(w).cuda()
+    assert torch.equal(mod.get_weight().view(torch.int16), w.view(torch.int16))
+    ratio = sum(b.numel() * b.element_size() for b in mod.buffers()) / (2 * M * K)
+    # short tasks (7 steps for 4608x3584) pay the 64-bit rANS state flush per lane
+    assert ratio < (0.75 if algo == "huffman" else 0.78), ratio
+    for bs in (1, 8):
+        x = torch.randn(bs, K, generator=g, device="cuda").bfloat16()
+        y = torch.nn.functional.linear(x, mod)
+        ref = x.float() @ w.float().T
+        torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
