@@ -25,6 +25,8 @@ _SIGNATURES = {
     "bhi_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_ans_encode": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp]),
     "bhi_ans_encode_capacity": (_i64, [_i32]),
+    "bhi_reference_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "bhi_reference_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
 }
 
 EXPORTS = tuple(_SIGNATURES)

@@ -38,6 +38,7 @@ __all__ = [
     "CompressedLinear",
     "convert_all_linear",
     "convert",
+    "load_compressed_state_dict",
 ]
 
 
@@ -346,6 +347,35 @@ def convert_all_linear(model: nn.Module, min_out_features=4096, progress=True, a
                if isinstance(m, nn.Linear) and m.out_features >= min_out_features]
     for name in tqdm(targets, disable=not progress):
         model.set_submodule(name, convert(model.get_submodule(name), name, algo=algo))
+
+
+def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool = True):
+    """Load the ``state_dict()`` of a converted model into a freshly built, unconverted one.
+
+    The reference leaves this to the user (its converted modules only exist after
+    ``convert_all_linear`` has run on real weights).  Here every ``nn.Linear`` of ``model``
+    whose compressed buffers are in ``state_dict`` (``<name>.weight.rem`` ...) is replaced
+    by a :class:`CompressedLinear` around those tensors -- ``LUT1`` present means Huffman,
+    ``LUT`` means rANS -- and the remaining entries go through ``load_state_dict``.  The
+    skeleton's linears may live on the meta device; nothing is decoded or re-encoded.
+    """
+    huffman_keys = ('rem', 'exp', 'offsets', 'LUT1', 'LUT2', 'LUT3', 'LUT4', 'code_lengths')
+    ans_keys = ('rem', 'exp', 'offsets', 'LUT')
+    for name, module in list(model.named_modules()):
+        if not isinstance(module, nn.Linear) or f'{name}.weight.rem' not in state_dict:
+            continue
+        keys = huffman_keys if f'{name}.weight.LUT1' in state_dict else ans_keys
+        cls = HuffmanWeight if keys is huffman_keys else ANSWeight
+        weight = cls(**{k: state_dict[f'{name}.weight.{k}'] for k in keys})
+        split_k, M, Ks = weight.rem.shape
+        if (M, split_k * Ks) != (module.out_features, module.in_features):
+            raise RuntimeError(f'{name}: compressed weight is {M}x{split_k * Ks}, '
+                               f'the module expects {module.out_features}x{module.in_features}')
+        bias = state_dict.get(f'{name}.bias')
+        if bias is not None:
+            bias = nn.Parameter(bias, requires_grad=False)
+        model.set_submodule(name, CompressedLinear(weight=weight, bias=bias))
+    return model.load_state_dict(state_dict, strict=strict, assign=True)
 
 
 def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tensor], fused) -> Tensor:

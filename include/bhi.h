@@ -112,6 +112,21 @@ int bhi_ans_encode(const void* data, const void* freq, const void* cum,
 
 int64_t bhi_ans_encode_capacity(int n_steps);
 
+/* Readers for weights that were compressed by the reference package itself: same tensors
+ * as the reference's huffman_decode / ans_decode ops (kernel.cu:534-587, 878-919) IN THE
+ * REFERENCE'S OWN LAYOUT (functional.py:129-242: 64 streams per row, LUT1..4 uint8 [256],
+ * code_lengths uint8 [256]; rANS LUT int32 [256]).  Y bf16 [M, split_k*Ks] receives the
+ * original weight, which can then be compressed again in this library's layout.  Only
+ * M >= 1 and Ks % 128 == 0 are required. */
+int bhi_reference_huffman_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
+                                 void* Y, const void* offsets,
+                                 const void* LUT1, const void* LUT2, const void* LUT3, const void* LUT4,
+                                 const void* code_lengths,
+                                 int split_k, int M, int Ks, void* stream);
+int bhi_reference_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
+                             void* Y, const void* offsets, const void* LUT,
+                             int split_k, int M, int Ks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -91,3 +91,35 @@ def test_convert_picks_codec_and_is_lossless(cuda, algo):
         assert type(out.weight) is min(sizes, key=sizes.get)
     out = out.cuda()
     assert torch.equal(out.weight.get_weight().view(torch.int16).cpu(), ref.view(torch.int16))
+
+
+def test_state_dict_of_a_converted_model_loads_into_a_fresh_one(cuda):
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight, convert, load_compressed_state_dict
+
+    def make():
+        torch.manual_seed(4)
+        return torch.nn.Sequential(torch.nn.Linear(512, 384, bias=True), torch.nn.SiLU(),
+                                   torch.nn.Linear(384, 256, bias=False), torch.nn.LayerNorm(256)).bfloat16()
+
+    model = make()
+    with torch.no_grad():
+        model[0].weight.copy_(gaussian_weight(384, 512, seed=1))
+        model[2].weight.copy_(student_t_weight(256, 384, seed=2))
+    x = torch.randn(3, 512).bfloat16().cuda()
+    want_dense = model.cuda()(x)
+    model.cpu()
+    model[0] = convert(model[0], "0", algo="huffman")
+    model[2] = convert(model[2], "2", algo="ans")
+    assert isinstance(model[0].weight, HuffmanWeight) and isinstance(model[2].weight, ANSWeight)
+    sd = {k: v.clone() for k, v in model.state_dict().items()}
+    assert "0.weight.rem" in sd and "2.weight.LUT" in sd and "0.bias" in sd
+    want = model.cuda()(x)
+
+    with torch.device("meta"):
+        fresh = make()
+    missing = load_compressed_state_dict(fresh, sd)
+    assert not missing.missing_keys and not missing.unexpected_keys
+    assert isinstance(fresh[0].weight, HuffmanWeight) and isinstance(fresh[2].weight, ANSWeight)
+    got = fresh.cuda()(x)
+    assert torch.equal(got, want)
+    torch.testing.assert_close(got.float(), want_dense.float(), rtol=5e-2, atol=5e-2)
