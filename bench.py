@@ -210,6 +210,8 @@ def main():
         "compressed_bytes_per_step": block_bytes, "compression_ratio": round(
             sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),
         "block_steps_per_s": round(1.0 / sec, 1),
+        # 28 such blocks make one Qwen2.5-7B token (attention, norms, embedding and lm_head not included)
+        "bs1_tokens_per_s_28_blocks": round(1.0 / sec / 28, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
         "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{'HuffCodec' if args.algo == 'huffman' else 'AnsCodec'}, {bs}, 4> "
                                f"18944x3584",

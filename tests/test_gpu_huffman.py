@@ -123,3 +123,25 @@ def test_full_size_layers_round_trip(cuda, algo, kind, M, K):
         y = torch.nn.functional.linear(x, mod)
         ref = x.float() @ w.float().T
         torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+def test_long_incompressible_tasks_outrun_the_row_ring(cuda, algo):
+    """128-step tasks whose exponents are uniform over 39 values: every pair costs about
+    10.6 bits, lanes consume rows faster than a segment stages them, so windows have to be
+    read from global memory behind the staged rows.  Decode and GEMV must not care."""
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight
+    g = torch.Generator().manual_seed(21)
+    M, K = 128, 16384
+    exp = torch.randint(90, 129, (M, K), generator=g, dtype=torch.int32)
+    rem = torch.randint(0, 256, (M, K), generator=g, dtype=torch.int32)
+    bits = ((rem << 8) & 0x8000) | (rem & 0x7F) | (exp << 7)
+    w = bits.to(torch.int16).view(torch.bfloat16)
+    mod = (HuffmanWeight if algo == "huffman" else ANSWeight).compress_split_n(w, n=1).cuda()
+    words_per_lane_step = (mod.exp.numel() - 2048) / (M // 4 * 128 * 64)
+    assert words_per_lane_step > 1.05, "the input no longer outruns the ring"
+    assert torch.equal(mod.get_weight().view(torch.int16).cpu(), w.view(torch.int16))
+    x = torch.randn(3, K, generator=g).bfloat16().cuda()
+    y = torch.nn.functional.linear(x, mod)
+    ref = x.float() @ w.cuda().float().T
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
