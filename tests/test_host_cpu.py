@@ -51,3 +51,24 @@ def test_compressed_ops_refuse_cpu_tensors():
     w = _huffman_weight(128, 384)
     with pytest.raises((AssertionError, RuntimeError, NotImplementedError)):
         torch.nn.functional.linear(torch.zeros(1, 384, dtype=torch.bfloat16), w)
+
+
+def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
+    """There is no fallback: without the built HIP library nothing of the package runs."""
+    from bf16_huffman_infer_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libbhi_hip.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.load()
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.constants()
+
+
+def test_package_does_not_import_the_oracle():
+    import subprocess
+    import sys
+    code = ("import sys, bf16_huffman_infer_amd, bf16_huffman_infer_amd.cudagraph_utils, "
+            "bf16_huffman_infer_amd.reference_format; "
+            "assert not [m for m in sys.modules if m == 'oracle' or m.startswith('oracle.')]")
+    subprocess.run([sys.executable, "-c", code], check=True, cwd=__import__("os").path.dirname(
+        __import__("os").path.dirname(__import__("os").path.abspath(__file__))))
