@@ -216,29 +216,25 @@ struct RowRing {
 
     // The lane's window: rows m, m+1, m+2 with m = pos >> 5.
     __device__ __forceinline__ void window(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
-        if (__builtin_expect(ballot(pos >= lim) != 0, 0)) {
-            fetch_slow(lo, hi, nx);
-        } else {
-            const lds_u32* w = slot_of(pos);
-            lo = w[0];
-            hi = w[kLanes];
-            nx = w[2 * kLanes];
-        }
+        // the ring is read unconditionally (a slot address is always valid); lanes whose
+        // window is not staged there get it from global memory instead
+        const lds_u32* w = slot_of(pos);
+        lo = w[0];
+        hi = w[kLanes];
+        nx = w[2 * kLanes];
+        if (__builtin_expect(ballot(pos >= lim) != 0, 0)) fetch_behind(lo, hi, nx);
     }
 
     // Some lane's window is not staged (it ran more than a ring ahead of the slowest lane,
-    // or further than one segment's prefetch): those lanes read global memory.
-    __device__ __forceinline__ void fetch_slow(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
-        const uint32_t m = pos >> 5;
+    // or faster than the segments stage rows): those lanes read global memory.  The
+    // address is kept in range for the others (the stream ends in a zero pad anyway).
+    __device__ __forceinline__ void fetch_behind(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
         const bool staged = pos < lim;
-        // both reads are always in range (the stream ends in a zero pad), then pick per lane
-        const lds_u32* w = slot_of(pos);
-        const uint32_t l0 = w[0], l1 = w[kLanes], l2 = w[2 * kLanes];
-        const uint32_t* g = bp + (size_t)(staged ? 0u : m) * kLanes;
+        const uint32_t* g = bp + (size_t)(staged ? 0u : pos >> 5) * kLanes;
         const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
-        lo = staged ? l0 : g0;
-        hi = staged ? l1 : g1;
-        nx = staged ? l2 : g2;
+        lo = staged ? lo : g0;
+        hi = staged ? hi : g1;
+        nx = staged ? nx : g2;
     }
 };
 
