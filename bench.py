@@ -48,8 +48,8 @@ def gemv_bytes(mod, bs, M, K) -> int:
 
 
 def build_block(algo, device, copy):
-    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight
-    cls = {"huffman": HuffmanWeight, "ans": ANSWeight}[algo]
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight, NibbleWeight
+    cls = {"huffman": HuffmanWeight, "ans": ANSWeight, "nibble": NibbleWeight}[algo]
     mods = []
     for i, (name, M, K) in enumerate(LAYERS):
         w = make_weight(M, K, 1000 * copy + i, device)
@@ -128,7 +128,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=1)
-    ap.add_argument("--algo", default="huffman", choices=["huffman", "ans"])
+    ap.add_argument("--algo", default="huffman", choices=["huffman", "ans", "nibble"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -213,7 +213,7 @@ def main():
         # 28 such blocks make one Qwen2.5-7B token (attention, norms, embedding and lm_head not included)
         "bs1_tokens_per_s_28_blocks": round(1.0 / sec / 28, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
-        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{'HuffCodec' if args.algo == 'huffman' else 'AnsCodec'}, {bs}, 4> "
+        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{dict(huffman='HuffCodec', ans='AnsCodec', nibble='NibbleCodec')[args.algo]}, {bs}, 4> "
                                f"18944x3584",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),

@@ -25,6 +25,10 @@ _SIGNATURES = {
     "bhi_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_ans_encode": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp]),
     "bhi_ans_encode_capacity": (_i64, [_i32]),
+    "bhi_gemv_bf16_nibble": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp]),
+    "bhi_nibble_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "bhi_nibble_encode": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp]),
+    "bhi_nibble_encode_capacity": (_i64, [_i32]),
     "bhi_reference_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_reference_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
 }

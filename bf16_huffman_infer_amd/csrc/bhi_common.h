@@ -264,11 +264,11 @@ struct HuffCursor : RowRing {
         eptr = 0;
     }
 
-    __device__ __forceinline__ void start() {}
+    __device__ __forceinline__ void start(const uint32_t*) {}
 
     // Decode the four pairs of one step; e[q] are raw table entries.
     template <bool HAS_ESC>
-    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
+    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4], int) {
         uint32_t lo, hi, nx;
         window(lo, hi, nx);
         const char* tb = (const char*)table;
@@ -316,7 +316,7 @@ struct AnsCursor : RowRing {
     }
 
     // rows 0 and 1 are the initial state (call after prime())
-    __device__ __forceinline__ void start() {
+    __device__ __forceinline__ void start(const uint32_t*) {
         xl = ring[0];
         xh = ring[kLanes];
         pos = 2 * 32;
@@ -349,7 +349,7 @@ struct AnsCursor : RowRing {
     }
 
     template <bool UNUSED>
-    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4]) {
+    __device__ __forceinline__ void step(const uint32_t* __restrict__ table, uint32_t (&e)[4], int) {
         uint32_t lo, hi, nx;
         window(lo, hi, nx);
         e[0] = pair(table);
@@ -359,6 +359,77 @@ struct AnsCursor : RowRing {
         e[2] = pair(table);
         e[3] = pair(table);
         refill(first ? hi : lo);
+    }
+};
+
+// Fixed-width exponent code: the eight nibbles of a lane and step sit in one word of the
+// task block's row t (column j in bits 4j..4j+3); a nibble is the exponent's offset from
+// `base`, 15 marks an exponent that travels in the escape list instead.  Nothing here
+// is sequential: the cursor only hands out the words the segment prefetched.  It has
+// the interface of the entropy cursors so that the same task walk drives it; the LDS
+// ring is not used.
+struct NibbleCursor {
+    const uint32_t* bp;      // task block, this lane's column
+    const uint32_t* ep;      // one past the task block (escape list grows down from here)
+    uint32_t eptr;           // wave-uniform: escape entries consumed so far
+    uint32_t next;           // wave-uniform: first step not prefetched yet
+    uint32_t base4;          // wave-uniform: the base exponent in every byte
+    uint32_t cur[kSegSteps]; // the words of the segment being decoded
+
+    __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t*) {
+        bp = words + span.base + lane;
+        ep = words + span.end;
+        eptr = 0;
+        next = 0;
+    }
+    __device__ __forceinline__ void prime() const {}
+    __device__ __forceinline__ void start(const uint32_t* lut) { base4 = uniform(lut[0] & 0xFFu) * 0x01010101u; }
+    __device__ __forceinline__ bool room() const { return true; }
+    static_assert(kSegRows == kSegSteps, "one row per step");
+
+    // rows past the last step belong to the escape list, the next block or the zero pad
+    __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) const {
+        const uint32_t* p = bp + (size_t)next * kLanes;
+#pragma unroll
+        for (int j = 0; j < kSegRows; ++j) v[j] = p[j * kLanes];
+    }
+    __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
+#pragma unroll
+        for (int j = 0; j < kSegRows; ++j) cur[j] = v[j];
+        next += kSegRows;
+    }
+
+    // pair entries in the Huffman table's format (a<<7 | b<<23) for step i of the segment
+    template <bool HAS_ESC>
+    __device__ __forceinline__ void step(const uint32_t*, uint32_t (&e)[4], int i) {
+        const uint32_t d = cur[i];
+        uint32_t even = (d & 0x0F0F0F0Fu) + base4;            // exponents of columns 0, 2, 4, 6
+        uint32_t odd = ((d >> 4) & 0x0F0F0F0Fu) + base4;      // exponents of columns 1, 3, 5, 7
+        if (HAS_ESC) {
+            uint32_t t = d & (d >> 1);
+            t &= t >> 2;                                       // bit 4j set iff nibble j is 15
+            if (__builtin_expect(ballot((t & 0x11111111u) != 0) != 0, 0)) escapes(t, even, odd);
+        }
+        e[0] = __builtin_amdgcn_perm(odd, even, 0x0C040C00u) << 7;
+        e[1] = __builtin_amdgcn_perm(odd, even, 0x0C050C01u) << 7;
+        e[2] = __builtin_amdgcn_perm(odd, even, 0x0C060C02u) << 7;
+        e[3] = __builtin_amdgcn_perm(odd, even, 0x0C070C03u) << 7;
+    }
+
+    // escaped exponents come from the escape list, in (column, lane) order
+    __device__ __forceinline__ void escapes(uint32_t t, uint32_t& even, uint32_t& odd) {
+#pragma unroll
+        for (int j = 0; j < kLaneCols; ++j) {
+            const bool esc = ((t >> (4 * j)) & 1u) != 0;
+            const uint64_t m = ballot(esc);
+            if (esc) {
+                const uint32_t raw = *(ep - 1 - (eptr + lane_rank(m))) & 0xFFu;
+                uint32_t& half = (j & 1) ? odd : even;
+                const int sh = 8 * (j >> 1);
+                half = (half & ~(0xFFu << sh)) | (raw << sh);
+            }
+            eptr = uniform(eptr + (uint32_t)__builtin_popcountll(m));
+        }
     }
 };
 

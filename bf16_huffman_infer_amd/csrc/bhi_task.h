@@ -44,7 +44,7 @@ __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut,
         if (FULL || t0 + i < ns) {
             const typename Policy::Piped piped = pol.take(slot[i], i, t0 + i);
             uint32_t e[4];
-            cur.template step<HAS_ESC>(lut, e);
+            cur.template step<HAS_ESC>(lut, e, i);
             uint32_t w[4];
             const uint2 r = slot[i].rem;
             w[0] = rebuild_pair(e[0], rem_lo_pair(r.x));
@@ -62,7 +62,7 @@ template <bool HAS_ESC, class Cursor, class Policy>
 __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns) {
     pol.prime();
     cur.prime();
-    cur.start();
+    cur.start(lut);
     typename Policy::Slot slot[kSegSteps];
     uint32_t rows[kSegRows];
     int seg = 0;

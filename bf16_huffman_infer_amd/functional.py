@@ -19,7 +19,8 @@ from . import _lib
 from .ans import RANSEncoder
 from .huffman import LUTHuffmanEncoder
 from .ops import (ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemv_bf16_ans,
-                  gemv_bf16_huffman, huffman_decode, huffman_encode)
+                  gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode, nibble_decode,
+                  nibble_encode, nibble_encode_capacity)
 from .utils import get_block_size_n, split_bf16
 
 ANS_PRECISION = 8
@@ -33,8 +34,10 @@ ENCODE_PART_BYTES = 256 << 20       # scratch bound per encode call
 __all__ = [
     "linear_huffman",
     "linear_ans",
+    "linear_nibble",
     "HuffmanWeight",
     "ANSWeight",
+    "NibbleWeight",
     "CompressedLinear",
     "convert_all_linear",
     "convert",
@@ -281,6 +284,65 @@ class ANSWeight(HuffmanWeight):
         return out, lengths
 
 
+class NibbleCodec:
+    """Per-matrix parameters of the fixed-width code: the start of the 15-wide exponent
+    window that covers the most weights, and whether anything falls outside it."""
+
+    WINDOW = 15
+
+    def __init__(self, counts: Tensor):
+        counts = counts.to(torch.int64).cpu()
+        assert counts.numel() == 256
+        cover = counts.unfold(0, self.WINDOW, 1).sum(-1)          # cover[b] = counts[b : b + 15]
+        self.base = int(torch.argmax(cover).item())               # first best window
+        self.has_escapes = int(cover[self.base].item()) != int(counts.sum().item())
+
+
+class NibbleWeight(ANSWeight):
+    """Same planes and task layout with a fixed-width exponent code: 4 bits per exponent
+    (offset from a per-matrix base, escape list for outliers).  Not one of the reference's
+    codecs: about nine percent larger than the Huffman form and noticeably faster to
+    multiply with, because its decoder has no tables, cursors or serial dependencies."""
+
+    MAGIC = 0x4E494242          # LUT[2]: tells this module's LUT from a rANS slot table (whose frequency field is <= 256)
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        if func is not F.linear:
+            return NotImplemented
+        return linear_nibble(*args, **(kwargs or {}))
+
+    def get_weight(self) -> Tensor:
+        weight = self._empty_weight()
+        nibble_decode(self.rem, self.exp, weight, self.offsets, self.LUT)
+        return weight
+
+    @classmethod
+    def get_codec(cls, a: Tensor) -> NibbleCodec:
+        device = torch.device('cuda', 0)
+        _, exp = split_bf16(a.detach().to(device))
+        return NibbleCodec(torch.bincount(exp.flatten().to(torch.int32), minlength=256))
+
+    @classmethod
+    def get_lut_kwargs(cls, codec: NibbleCodec) -> dict[str, Tensor]:
+        lut = torch.zeros(256, dtype=torch.int32)
+        lut[0], lut[1], lut[2] = codec.base, int(codec.has_escapes), cls.MAGIC
+        return {'LUT': lut}
+
+    @classmethod
+    def capacity(cls, n_steps: int) -> int:
+        return nibble_encode_capacity(n_steps)
+
+    @classmethod
+    def compress_groups(cls, x: Tensor, codec: NibbleCodec) -> tuple[Tensor, Tensor]:
+        device = x.device
+        n_steps = x.size(1) // (LANES * LANE_COLS)
+        out = torch.zeros(x.size(0), cls.capacity(n_steps), dtype=torch.int32, device=device)
+        lengths = torch.zeros(x.size(0), dtype=torch.int32, device=device)
+        nibble_encode(x, cls.get_lut_kwargs(codec)['LUT'].to(device), out, lengths)
+        return out, lengths
+
+
 class CompressedLinear(nn.Module):
     def __init__(self, weight: HuffmanWeight, bias: Optional[Tensor]) -> None:
         super().__init__()
@@ -302,11 +364,13 @@ def convert(linear: nn.Linear, name, disable_precision_check=True, algo='huffman
     weight is not bit-identical; with ``disable_precision_check=False`` also when one
     random GEMV deviates by 2 % or more from the dense layer.
     """
-    assert algo in ('huffman', 'ans', 'smallest')
+    assert algo in ('huffman', 'ans', 'smallest', 'nibble')
     if algo == 'huffman':
         weight = HuffmanWeight.compress(linear.weight)
     elif algo == 'ans':
         weight = ANSWeight.compress(linear.weight)
+    elif algo == 'nibble':
+        weight = NibbleWeight.compress(linear.weight)
     else:
         weight = min([HuffmanWeight.compress(linear.weight), ANSWeight.compress(linear.weight)], key=_weight_bytes)
 
@@ -349,6 +413,18 @@ def convert_all_linear(model: nn.Module, min_out_features=4096, progress=True, a
         model.set_submodule(name, convert(model.get_submodule(name), name, algo=algo))
 
 
+def linear_nibble(input: Tensor, weight: NibbleWeight, bias: Optional[Tensor] = None) -> Tensor:
+    """``F.linear`` with a :class:`NibbleWeight` (fused up to 8 rows, else decode + GEMM)."""
+    def fused(x):
+        split_k, M, N = weight.rem.shape
+        x = x.view(-1, split_k, N)
+        _check_weight_call(weight.rem, weight.exp, x)
+        y = torch.empty((x.size(0), M), dtype=torch.bfloat16, device=x.device)
+        gemv_bf16_nibble(weight.rem, weight.exp, x.contiguous(), y, weight.offsets, weight.LUT)
+        return y
+    return _linear_compressed(input, weight, bias, fused)
+
+
 def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool = True):
     """Load the ``state_dict()`` of a converted model into a freshly built, unconverted one.
 
@@ -356,7 +432,7 @@ def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool 
     ``convert_all_linear`` has run on real weights).  Here every ``nn.Linear`` of ``model``
     whose compressed buffers are in ``state_dict`` (``<name>.weight.rem`` ...) is replaced
     by a :class:`CompressedLinear` around those tensors -- ``LUT1`` present means Huffman,
-    ``LUT`` means rANS -- and the remaining entries go through ``load_state_dict``.  The
+    ``LUT`` means rANS or (by its marker word) the nibble code -- and the remaining entries go through ``load_state_dict``.  The
     skeleton's linears may live on the meta device; nothing is decoded or re-encoded.
     """
     huffman_keys = ('rem', 'exp', 'offsets', 'LUT1', 'LUT2', 'LUT3', 'LUT4', 'code_lengths')
@@ -365,7 +441,11 @@ def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool 
         if not isinstance(module, nn.Linear) or f'{name}.weight.rem' not in state_dict:
             continue
         keys = huffman_keys if f'{name}.weight.LUT1' in state_dict else ans_keys
-        cls = HuffmanWeight if keys is huffman_keys else ANSWeight
+        if keys is huffman_keys:
+            cls = HuffmanWeight
+        else:
+            nibble = int(state_dict[f'{name}.weight.LUT'][2]) == NibbleWeight.MAGIC
+            cls = NibbleWeight if nibble else ANSWeight
         weight = cls(**{k: state_dict[f'{name}.weight.{k}'] for k in keys})
         split_k, M, Ks = weight.rem.shape
         if (M, split_k * Ks) != (module.out_features, module.in_features):

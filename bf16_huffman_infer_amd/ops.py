@@ -1,4 +1,4 @@
-"""The six custom ops of namespace ``bf16_huffman_infer`` on HIP.
+"""The six custom ops of namespace ``bf16_huffman_infer`` on HIP (plus three for the nibble codec).
 
 Same op names, schemas and positional wrappers as the reference
 (``bf16_huffman_infer/src/bf16_huffman_infer.cpp:29-35``, ``ops.py:6-61``).  The schemas
@@ -24,6 +24,10 @@ _LIB.define("huffman_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor off
 _LIB.define("gemv_bf16_ans(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
 _LIB.define("ans_encode(Tensor data, Tensor freq, Tensor cum, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
 _LIB.define("ans_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
+# not in the reference: the fixed-width codec, with the rANS ops' shapes
+_LIB.define("gemv_bf16_nibble(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
+_LIB.define("nibble_encode(Tensor data, Tensor LUT, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
+_LIB.define("nibble_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
 
 LANE_BYTES_PER_STEP = 512          # 64 lanes x 8 exponent bytes
 
@@ -156,6 +160,52 @@ def _ans_encode(data, freq, cum, output, output_lengths):
     _lib.check(rc, "ans_encode")
 
 
+def _gemv_bf16_nibble(A_rem, A_exp, X, Y, offsets, LUT):
+    lib = _lib.load()
+    split_k, M, Ks, batch = _gemv_common(A_rem, A_exp, X, Y, offsets)
+    if LUT.numel() != 256:
+        raise RuntimeError("LUT must hold 256 entries")
+    with torch.cuda.device(A_rem.device):
+        rc = lib.bhi_gemv_bf16_nibble(
+            _req(A_rem, torch.uint8, "A_rem"), _req(A_exp, torch.int32, "A_exp", A_rem), A_exp.numel(),
+            _req(X, torch.bfloat16, "X", A_rem), _req(Y, torch.bfloat16, "Y", A_rem),
+            _req(offsets, torch.int32, "offsets", A_rem), _req(LUT, torch.int32, "LUT", A_rem),
+            split_k, M, Ks, batch, _stream(A_rem))
+    _lib.check(rc, "gemv_bf16_nibble")
+
+
+def _nibble_decode(A_rem, A_exp, Y, offsets, LUT):
+    lib = _lib.load()
+    split_k, M, Ks = _weight_dims(A_rem, offsets)
+    if tuple(Y.shape) != (M, split_k * Ks):
+        raise RuntimeError(f"Y must be [{M}, {split_k * Ks}], got {tuple(Y.shape)}")
+    if LUT.numel() != 256:
+        raise RuntimeError("LUT must hold 256 entries")
+    with torch.cuda.device(A_rem.device):
+        rc = lib.bhi_nibble_decode(
+            _req(A_rem, torch.uint8, "A_rem"), _req(A_exp, torch.int32, "A_exp", A_rem), A_exp.numel(),
+            _req(Y, torch.bfloat16, "Y", A_rem), _req(offsets, torch.int32, "offsets", A_rem),
+            _req(LUT, torch.int32, "LUT", A_rem), split_k, M, Ks, _stream(A_rem))
+    _lib.check(rc, "nibble_decode")
+
+
+def _nibble_encode(data, LUT, output, output_lengths):
+    lib = _lib.load()
+    n_tasks, n_steps = _encode_dims(data, output, output_lengths)
+    if LUT.numel() != 256:
+        raise RuntimeError("LUT must hold 256 entries")
+    with torch.cuda.device(data.device):
+        rc = lib.bhi_nibble_encode(
+            _req(data, torch.uint8, "data"), _req(LUT, torch.int32, "LUT", data),
+            _req(output, torch.int32, "output", data), _req(output_lengths, torch.int32, "output_lengths", data),
+            n_tasks, n_steps, output.shape[1], _stream(data))
+    _lib.check(rc, "nibble_encode")
+
+
+for _name, _fn in (("gemv_bf16_nibble", _gemv_bf16_nibble), ("nibble_encode", _nibble_encode),
+                   ("nibble_decode", _nibble_decode)):
+    _LIB.impl(_name, _fn, "CUDA")
+
 for _name, _fn in (("gemv_bf16_huffman", _gemv_bf16_huffman), ("huffman_encode", _huffman_encode),
                    ("huffman_decode", _huffman_decode), ("gemv_bf16_ans", _gemv_bf16_ans),
                    ("ans_encode", _ans_encode), ("ans_decode", _ans_decode)):
@@ -205,3 +255,19 @@ def encode_capacity(n_steps: int) -> int:
 
 def ans_encode_capacity(n_steps: int) -> int:
     return int(_lib.load().bhi_ans_encode_capacity(n_steps))
+
+
+def gemv_bf16_nibble(A_rem: Tensor, A_exp: Tensor, X: Tensor, Y: Tensor, offsets: Tensor, LUT: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.gemv_bf16_nibble.default(A_rem, A_exp, X, Y, offsets, LUT)
+
+
+def nibble_encode(data: Tensor, LUT: Tensor, output: Tensor, output_lengths: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.nibble_encode.default(data, LUT, output, output_lengths)
+
+
+def nibble_decode(A_rem: Tensor, A_exp: Tensor, Y: Tensor, offsets: Tensor, LUT: Tensor) -> None:
+    torch.ops.bf16_huffman_infer.nibble_decode.default(A_rem, A_exp, Y, offsets, LUT)
+
+
+def nibble_encode_capacity(n_steps: int) -> int:
+    return int(_lib.load().bhi_nibble_encode_capacity(n_steps))

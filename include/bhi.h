@@ -112,6 +112,21 @@ int bhi_ans_encode(const void* data, const void* freq, const void* cum,
 
 int64_t bhi_ans_encode_capacity(int n_steps);
 
+/* Fixed-width ("nibble") codec -- no counterpart in the reference.  Every exponent inside
+ * [base, base+14] is a 4-bit offset in the task block's rows (row t = step t, column j in
+ * bits 4j..4j+3 of the lane's word), nibble 15 sends the exponent to the block's escape
+ * list.  Same tensors and meanings as the rANS entry points; LUT int32 [256]: [0] base
+ * exponent, [1] nonzero when the matrix has escaped exponents, the rest 0. */
+int bhi_gemv_bf16_nibble(const void* A_rem, const void* A_exp, int64_t exp_words,
+                         const void* X, void* Y, const void* offsets, const void* LUT,
+                         int split_k, int M, int Ks, int batch, void* stream);
+int bhi_nibble_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
+                      void* Y, const void* offsets, const void* LUT,
+                      int split_k, int M, int Ks, void* stream);
+int bhi_nibble_encode(const void* data, const void* LUT, void* output, void* output_lengths,
+                      int n_tasks, int n_steps, int64_t out_stride, void* stream);
+int64_t bhi_nibble_encode_capacity(int n_steps);
+
 /* Readers for weights that were compressed by the reference package itself: same tensors
  * as the reference's huffman_decode / ans_decode ops (kernel.cu:534-587, 878-919) IN THE
  * REFERENCE'S OWN LAYOUT (functional.py:129-242: 64 streams per row, LUT1..4 uint8 [256],

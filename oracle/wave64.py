@@ -390,6 +390,122 @@ def decode_ans(rem_packed: np.ndarray, exp_words: np.ndarray, offsets: np.ndarra
     return rebuild_bf16(unpack_rem(rem_packed), lane_order_inverse(sym))
 
 
+# ----------------------------------------------------------------------------- nibble codec
+#
+# A fixed-width code (not in the reference): every exponent inside a window of 15
+# consecutive values ``[base, base + 14]`` is stored as the 4-bit offset from ``base``,
+# anything else as the nibble 15 plus one word of the task's escape list.  Same planes,
+# tasks, lanes and offsets as the other codecs; a task block is
+# ``[ns rows of 64 words][escape list][zero pad]``: row ``t``, lane ``l`` holds the eight
+# nibbles of the lane's columns of step ``t`` (column ``j`` in bits ``4j..4j+3``).  Escape
+# words (the raw exponent) are consumed per step in (column, lane) order and stored
+# backwards from the end of the block.  Nothing is variable-length inside a block, so
+# the decoder needs no table, no cursor and no serial dependency.
+
+NIBBLE_ESC = 15
+
+
+def nibble_base(counts: np.ndarray) -> int:
+    """Start of the 15-wide exponent window that covers the most weights (first best)."""
+    c = np.asarray(counts, dtype=np.int64)
+    cover = np.convolve(c, np.ones(NIBBLE_ESC, dtype=np.int64))[NIBBLE_ESC - 1:NIBBLE_ESC - 1 + 256 - NIBBLE_ESC + 1]
+    return int(np.argmax(cover))
+
+
+def nibble_capacity(n_steps: int) -> int:
+    return n_steps * LANES + n_steps * LANE_COLS * LANES + ALIGN_WORDS
+
+
+def _nibble_encode_tasks(sym: np.ndarray, base: int):
+    """sym: uint8 [nt, ns, 64, 8] -> list of nt uint32 task blocks."""
+    nt, ns = sym.shape[:2]
+    off = sym.astype(np.int64) - base
+    esc = (off < 0) | (off >= NIBBLE_ESC)
+    nib = np.where(esc, NIBBLE_ESC, off).astype(np.uint32)
+    rows = np.zeros((nt, ns, LANES), dtype=np.uint32)
+    for j in range(LANE_COLS):
+        rows |= nib[..., j] << np.uint32(4 * j)
+    esc_flat = esc.transpose(0, 1, 3, 2).reshape(nt, -1)             # (step, column, lane) order
+    raw_flat = sym.transpose(0, 1, 3, 2).reshape(nt, -1).astype(np.uint32)
+    blocks = []
+    for t in range(nt):
+        nesc = int(esc_flat[t].sum())
+        total = (ns * LANES + nesc + ALIGN_WORDS - 1) // ALIGN_WORDS * ALIGN_WORDS
+        blk = np.zeros(total, dtype=np.uint32)
+        blk[:ns * LANES] = rows[t].reshape(-1)
+        if nesc:
+            blk[total - 1 - np.arange(nesc)] = raw_flat[t][esc_flat[t]]
+        blocks.append(blk)
+    return blocks
+
+
+def _nibble_decode_tasks(words: np.ndarray, base_w: np.ndarray, end_w: np.ndarray, ns: int, base: int) -> np.ndarray:
+    nt = len(base_w)
+    lanes = np.arange(LANES)
+    out = np.zeros((nt, ns, LANES, LANE_COLS), dtype=np.uint8)
+    eptr = np.zeros(nt, dtype=np.int64)
+    for t in range(ns):
+        d = words[base_w[:, None] + t * LANES + lanes]
+        for j in range(LANE_COLS):
+            n = (d >> np.uint32(4 * j)) & np.uint32(15)
+            esc = n == NIBBLE_ESC
+            val = (n + np.uint32(base)).astype(np.uint8)
+            if esc.any():
+                rank = np.cumsum(esc, axis=-1) - esc
+                src = end_w[:, None] - 1 - (eptr[:, None] + rank)
+                raw = words[np.where(esc, src, 0)]
+                val = np.where(esc, raw.astype(np.uint8), val)
+                eptr += esc.sum(axis=-1)
+            out[:, t, :, j] = val
+    return out
+
+
+def encode_nibble(bits: np.ndarray, split_k: int, base: int):
+    """bits: uint16 [M, K] BF16 patterns -> dict(rem, exp, offsets, nc)."""
+    from .planes import split_bf16
+    M, K = bits.shape
+    Ks = K // split_k
+    S, G = Ks // STEP_COLS, M // GROUP_ROWS
+    nc = chunks_per_group(M, Ks, split_k)
+    rem, exp = split_bf16(bits)
+    sym = lane_order(exp, split_k)
+    per_chunk = []
+    for c in range(nc):
+        t0, t1 = chunk_steps(S, nc, c)
+        per_chunk.append(_nibble_encode_tasks(sym[:, :, t0:t1].reshape(split_k * G, t1 - t0, LANES, LANE_COLS), base))
+    offsets = np.zeros((split_k, M), dtype=np.int64)
+    parts, cursor = [], 0
+    for k in range(split_k):
+        for g in range(G):
+            for c in range(nc):
+                blk = per_chunk[c][k * G + g]
+                offsets[k, GROUP_ROWS * g + c] = cursor
+                parts.append(blk)
+                cursor += len(blk)
+    parts.append(np.zeros(TAIL_PAD_WORDS, dtype=np.uint32))
+    return {"rem": pack_rem(rem, split_k), "exp": np.concatenate(parts).view(np.int32),
+            "offsets": offsets.astype(np.int32), "nc": nc}
+
+
+def decode_nibble(rem_packed: np.ndarray, exp_words: np.ndarray, offsets: np.ndarray, base: int) -> np.ndarray:
+    """-> uint16 [M, K] BF16 patterns."""
+    from .planes import rebuild_bf16
+    split_k, M, Ks = rem_packed.shape
+    S, G = Ks // STEP_COLS, M // GROUP_ROWS
+    nc = chunks_per_group(M, Ks, split_k)
+    words = exp_words.view(np.uint32)
+    total = len(words) - TAIL_PAD_WORDS
+    off = offsets.astype(np.int64).reshape(split_k, G, GROUP_ROWS)[:, :, :nc]
+    flat = off.reshape(-1)
+    nxt = np.concatenate([flat[1:], [total]]).reshape(off.shape)
+    sym = np.zeros((split_k, G, S, LANES, LANE_COLS), dtype=np.uint8)
+    for c in range(nc):
+        t0, t1 = chunk_steps(S, nc, c)
+        r = _nibble_decode_tasks(words, off[:, :, c].reshape(-1), nxt[:, :, c].reshape(-1), t1 - t0, base)
+        sym[:, :, t0:t1] = r.reshape(split_k, G, t1 - t0, LANES, LANE_COLS)
+    return rebuild_bf16(unpack_rem(rem_packed), lane_order_inverse(sym))
+
+
 # ----------------------------------------------------------------------------- table checks
 
 def check_tables(dec: np.ndarray, enc: np.ndarray) -> None:

@@ -303,3 +303,39 @@ def test_ans_capacity_matches_library():
     lib = _lib.load()
     for ns in (1, 4, 28, 37, 128):
         assert lib.bhi_ans_encode_capacity(ns) == wave64.ans_capacity(ns)
+
+
+# ----------------------------------------------------------------------------- nibble codec in the wave64 layout
+
+@pytest.mark.parametrize("kind,M,K,n", [("gauss", 64, 1024, 1), ("t3", 32, 768, 2), ("bits", 16, 384, 1),
+                                        ("special", 32, 512, 1), ("zeros", 8, 384, 1)])
+def test_wave64_nibble_round_trip(kind, M, K, n):
+    makers = {"gauss": gaussian_weight, "t3": student_t_weight, "bits": random_bits_weight,
+              "special": special_values_weight, "zeros": lambda M, K, seed=0: torch.zeros(M, K, dtype=torch.bfloat16)}
+    bits = bits_of(makers[kind](M, K, seed=2))
+    _, exp = planes.split_bf16(bits)
+    base = wave64.nibble_base(np.bincount(exp.reshape(-1), minlength=256))
+    enc = wave64.encode_nibble(bits, n, base)
+    assert np.array_equal(wave64.decode_nibble(enc["rem"], enc["exp"], enc["offsets"], base), bits)
+    inside = ((exp >= base) & (exp < base + 15)).sum()
+    words = len(enc["exp"]) - wave64.TAIL_PAD_WORDS
+    assert words * 4 >= exp.size // 2 + 4 * (exp.size - inside)          # half a byte each + a word per outlier
+
+
+def test_nibble_base_is_the_first_best_window():
+    c = np.zeros(256, dtype=np.int64)
+    c[100:120] = np.arange(20)
+    assert wave64.nibble_base(c) == max(range(242), key=lambda b: (c[b:b + 15].sum(), -b)) == 105
+    c[:] = 1
+    assert wave64.nibble_base(c) == 0
+    from bf16_huffman_infer_amd.functional import NibbleCodec
+    for seed in range(3):
+        h = np.random.default_rng(seed).integers(0, 1000, 256)
+        assert NibbleCodec(torch.from_numpy(h)).base == wave64.nibble_base(h)
+
+
+def test_nibble_capacity_matches_library():
+    from bf16_huffman_infer_amd import _lib
+    lib = _lib.load()
+    for ns in (1, 4, 28, 37, 128):
+        assert lib.bhi_nibble_encode_capacity(ns) == wave64.nibble_capacity(ns)
