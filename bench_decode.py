@@ -182,7 +182,7 @@ def main():
     ap.add_argument("--layers", type=int, default=36)
     ap.add_argument("--tokens", type=int, default=256)
     ap.add_argument("--prompt", type=int, default=16)
-    ap.add_argument("--algo", default="smallest", choices=["huffman", "ans", "smallest"])
+    ap.add_argument("--algo", default="smallest", choices=["huffman", "ans", "smallest", "nibble"])
     ap.add_argument("--repeats", type=int, default=3)
     ap.add_argument("--small", action="store_true", help="tiny shapes (smoke run)")
     args = ap.parse_args()
@@ -214,7 +214,7 @@ def main():
     convert_s = time.time() - t0
     kinds = {}
     for m in model.modules():
-        if type(m).__name__ in ("HuffmanWeight", "ANSWeight"):
+        if type(m).__name__ in ("HuffmanWeight", "ANSWeight", "NibbleWeight"):
             kinds[type(m).__name__] = kinds.get(type(m).__name__, 0) + 1
     new_size = get_model_size(model)
     new_ids, new_s = best(model)

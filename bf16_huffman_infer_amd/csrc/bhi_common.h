@@ -238,18 +238,9 @@ struct RowRing {
     }
 };
 
-// The table entry selected by bits 2..13 of a (pre-shifted) window.
-#if defined(BHI_PROBE_SWZ)
-__device__ __forceinline__ uint32_t table_swizzle(uint32_t a) { return a ^ ((a >> 5) & 0x7Cu); }
-#else
-__device__ __forceinline__ uint32_t table_swizzle(uint32_t a) { return a; }
-#endif
+// The table entry selected by bits 2..12 of a (pre-shifted) window.
 __device__ __forceinline__ uint32_t table_entry(const char* tb, uint32_t w) {
-    const uint32_t a = table_swizzle(w & kTableMask);
-#if defined(BHI_PROBE_DUP)
-    (void)*(const volatile uint32_t*)(tb + (a ^ 0x1000u));
-#endif
-    return *(const uint32_t*)(tb + a);
+    return *(const uint32_t*)(tb + (w & kTableMask));
 }
 
 // Per-lane Huffman bit cursor.  pos = bit position - 2: the window is kept shifted left
@@ -388,15 +379,15 @@ struct NibbleCursor {
     static_assert(kSegRows == kSegSteps, "one row per step");
 
     // rows past the last step belong to the escape list, the next block or the zero pad
-    __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) const {
+    __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) {
         const uint32_t* p = bp + (size_t)next * kLanes;
 #pragma unroll
         for (int j = 0; j < kSegRows; ++j) v[j] = p[j * kLanes];
+        next += kSegRows;                          // segments are prefetched in order, possibly one ahead
     }
     __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
 #pragma unroll
         for (int j = 0; j < kSegRows; ++j) cur[j] = v[j];
-        next += kSegRows;
     }
 
     // pair entries in the Huffman table's format (a<<7 | b<<23) for step i of the segment

@@ -17,11 +17,7 @@ template <int WORDS>
 __device__ __forceinline__ void load_table(uint32_t* __restrict__ lds, const uint32_t* __restrict__ g) {
     const uint4* src = (const uint4*)g;
     uint4* dst = (uint4*)lds;
-#if defined(BHI_PROBE_SWZ)
-    for (int i = threadIdx.x; i < WORDS; i += blockDim.x) *(uint32_t*)((char*)lds + table_swizzle(4u * i)) = g[i];
-#else
     for (int i = threadIdx.x; i < WORDS / 4; i += blockDim.x) dst[i] = src[i];
-#endif
 }
 
 struct Shape {
