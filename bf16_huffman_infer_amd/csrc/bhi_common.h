@@ -87,18 +87,18 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
 }
 
 // A task is processed in segments of kSegSteps steps; the global loads of a segment (all
-// unconditional) are issued back to back before it is decoded.  VMEM loads complete in
-// issue order, so a load issued on demand inside a segment would make its wait drain the
-// whole queue.
+// unconditional) are issued back to back, one whole segment before they are used.  VMEM
+// loads complete in issue order, so a load issued on demand inside a segment would make
+// its wait drain the whole queue.
 //
 // Exponent rows are staged in a per-wavefront LDS ring of kRingRows rows (256 B each).
 // Row r lives in slot r % kRingRows; slots 0 and 1 are mirrored behind the last slot so
 // that the three rows of a window are always at +0, +256 and +512 bytes of one address.
 // Lanes sit at different rows, yet row r of lane l is always in bank l % 32: window reads
-// are conflict free.  Every segment prefetches
-// the next kSegRows rows and commits them to the ring before it is decoded if the
-// slowest lane has made room; a lane whose window is not staged (a cheap per-step test)
-// reads it from global memory instead.
+// are conflict free.  A task stages kPrimeRows rows before its first step; every segment
+// then prefetches the next kSegRows rows if every lane has made room for them, and the
+// following segment commits them to the ring.  A lane whose window is not staged (a
+// cheap per-step test) reads it from global memory instead.
 #ifndef BHI_SEG_STEPS
 #define BHI_SEG_STEPS 4
 #define BHI_SEG_ROWS 4
@@ -109,33 +109,19 @@ constexpr int kSegSteps = BHI_SEG_STEPS;
 #endif
 constexpr int kRingRows = BHI_RING_ROWS;
 constexpr int kSegRows = BHI_SEG_ROWS;          // rows prefetched per segment
+#ifndef BHI_PRIME_ROWS
+#define BHI_PRIME_ROWS 8
+#endif
+constexpr int kPrimeRows = BHI_PRIME_ROWS;      // rows staged before the first step
 constexpr int kRingSlots = kRingRows + 2;   // slots 0 and 1 are mirrored behind the last one
 constexpr int kRingWords = kRingSlots * kLanes;
 static_assert(kRingRows % kSegRows == 0 && (kRingRows & (kRingRows - 1)) == 0 && kSegRows >= 2,
               "rows are committed in aligned groups; the group at slot 0 carries both mirrored rows");
+static_assert(kPrimeRows % kSegRows == 0 && kPrimeRows >= 4 && kPrimeRows <= kRingRows, "priming stages whole groups");
 
 // LDS pointers are kept in their own address space: a pointer that may be LDS or global
 // turns every access into a flat load, which waits on the global-memory counter.
 typedef __attribute__((address_space(3))) uint32_t lds_u32;
-
-// Minimum over the wavefront, on the cross-lane data path (no LDS traffic): shifts within
-// rows of 16 lanes leave each row's minimum in its lane 15, two row broadcasts carry it
-// on to lane 63.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint32_t dpp_min(uint32_t v) {
-    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xF, false);
-    return o < v ? o : v;
-}
-
-__device__ __forceinline__ uint32_t wave_min(uint32_t v) {
-    v = dpp_min<0x111, 0xF>(v);      // row_shr:1
-    v = dpp_min<0x112, 0xF>(v);      // row_shr:2
-    v = dpp_min<0x114, 0xF>(v);      // row_shr:4
-    v = dpp_min<0x118, 0xF>(v);      // row_shr:8
-    v = dpp_min<0x142, 0xA>(v);      // row_bcast:15 into rows 1 and 3
-    v = dpp_min<0x143, 0xC>(v);      // row_bcast:31 into rows 2 and 3
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
 
 // A lane's view of its task block: a bit position in its own column of rows, and the
 // wavefront's LDS ring of staged rows.  The codec cursors below build on it.
@@ -161,20 +147,22 @@ struct RowRing {
         return ring + ((p >> 5) & (kRingRows - 1)) * kLanes;
     }
 
-    // Stage the first kRingRows rows of the block (once per task; the loads are waited for
-    // here).  Rows past the end of a short block are filler nobody decodes.
-    __device__ __forceinline__ void prime() {
-        uint32_t v[kRingRows];
+    // Stage the first kRingRows rows of the block, once per task, in two halves so that the
+    // caller can put other work between the loads and their use.  Rows past the end of a
+    // short block are filler nobody decodes.
+    __device__ __forceinline__ void prime_issue(uint32_t (&v)[kPrimeRows]) const {
 #pragma unroll
-        for (int j = 0; j < kRingRows; ++j) {
+        for (int j = 0; j < kPrimeRows; ++j) {
             const uint32_t r = (uint32_t)j < nrows ? (uint32_t)j : nrows - 1;
             v[j] = bp[(size_t)r * kLanes];
         }
+    }
+    __device__ __forceinline__ void prime_commit(const uint32_t (&v)[kPrimeRows]) {
 #pragma unroll
-        for (int j = 0; j < kRingRows; ++j) ring[j * kLanes] = v[j];
+        for (int j = 0; j < kPrimeRows; ++j) ring[j * kLanes] = v[j];
         ring[kRingRows * kLanes] = v[0];
         ring[(kRingRows + 1) * kLanes] = v[1];
-        rhi = kRingRows;
+        rhi = kPrimeRows;
         set_lim();
     }
 
@@ -184,13 +172,14 @@ struct RowRing {
     }
 
     // Can the next kSegRows rows be staged now?  Row r may replace row r - kRingRows once
-    // no window needs it, i.e. once the slowest lane is past it.  Rows are staged in whole
-    // groups: rhi stays a multiple of kSegRows and a group never wraps around the ring.
-    // Decided before the loads are issued so that they need not be issued in vain (and so
-    // that the compiler cannot sink them behind the decision, next to their use).
+    // no window needs it, i.e. once every lane is past it: one compare and a ballot.  Rows
+    // are staged in whole groups: rhi stays a multiple of kSegRows and a group never wraps
+    // around the ring.  Decided before the loads are issued so that they need not be
+    // issued in vain (and so that the compiler cannot sink them behind the decision).
     __device__ __forceinline__ bool room() const {
-        const uint32_t mmin = uniform(wave_min(pos)) >> 5;
-        return rhi < nrows && rhi + kSegRows <= mmin + kRingRows;
+        const uint32_t top = rhi + kSegRows;
+        const uint32_t oldest = top > (uint32_t)kRingRows ? (top - kRingRows) << 5 : 0u;
+        return rhi < nrows && ballot(pos < oldest) == 0;
     }
 
     // The next kSegRows rows after the staged ones: one address, immediate offsets.  Rows
@@ -232,6 +221,9 @@ struct RowRing {
         const bool staged = pos < lim;
         const uint32_t* g = bp + (size_t)(staged ? 0u : pos >> 5) * kLanes;
         const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
+        // vmcnt(0) here, inside the rare branch: otherwise the wait lands behind the join
+        // and every step would drain the operand loads that are in flight for later steps
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         lo = staged ? lo : g0;
         hi = staged ? hi : g1;
         nx = staged ? nx : g2;
@@ -306,7 +298,7 @@ struct AnsCursor : RowRing {
         open_rows(words, span, lane, ring_);
     }
 
-    // rows 0 and 1 are the initial state (call after prime())
+    // rows 0 and 1 are the initial state (call after prime_commit())
     __device__ __forceinline__ void start(const uint32_t*) {
         xl = ring[0];
         xh = ring[kLanes];
@@ -373,7 +365,8 @@ struct NibbleCursor {
         eptr = 0;
         next = 0;
     }
-    __device__ __forceinline__ void prime() const {}
+    __device__ __forceinline__ void prime_issue(uint32_t (&)[kPrimeRows]) const {}
+    __device__ __forceinline__ void prime_commit(const uint32_t (&)[kPrimeRows]) const {}
     __device__ __forceinline__ void start(const uint32_t* lut) { base4 = uniform(lut[0] & 0xFFu) * 0x01010101u; }
     __device__ __forceinline__ bool room() const { return true; }
     static_assert(kSegRows == kSegSteps, "one row per step");

@@ -25,13 +25,10 @@ struct Shape {
     uint32_t total_words;
 };
 
-// Runs one task in segments of kSegSteps steps: load phase (every global load of the
-// segment, unconditional), then decode.  A policy supplies the operands that travel with
-// the exponent stream: `Slot` holds what is loaded per step (`load(slot, t)`, t clamped by
-// the policy); `take(...)` hands out what the policy pipelines on its own inside the
-// compute phase; `use(...)` receives the lane's four rebuilt BF16 pairs (columns 0..7 of
-// its row in step t).  Because every load is unconditional the compiler can count the
-// outstanding ones and make each step wait for exactly its own operands.
+// One segment of a task: kSegSteps steps whose operands a policy has loaded into `slot`.
+// `Slot` holds what is loaded per step; `take(...)` hands out what the policy pipelines
+// on its own inside the compute phase; `use(...)` receives the lane's four rebuilt BF16
+// pairs (columns 0..7 of its row in step t).
 template <bool FULL, bool HAS_ESC, class Cursor, class Policy>
 __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut, Policy& pol,
                                                const typename Policy::Slot (&slot)[kSegSteps], int t0, int ns) {
@@ -52,31 +49,69 @@ __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut,
     }
 }
 
-// Whole segments load their operands from one address with immediate offsets and decode
-// without per-step guards; a last, shorter segment clamps its step indices instead.
+// A whole segment: stage the rows prefetched during the previous segment, prefetch the
+// next ones if the ring has room, issue the operand loads of the following segment into
+// `next`, decode `now`.  Every global load is thus issued a whole segment before its
+// first use and is unconditional apart from the row prefetch, so the compiler can count
+// the outstanding ones and make each step wait for exactly its own operands.
 template <bool HAS_ESC, class Cursor, class Policy>
-__device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns) {
+__device__ __forceinline__ void run_segment(Cursor& cur, const uint32_t* lut, Policy& pol, bool& pending,
+                                            uint32_t (&rows)[kSegRows], const typename Policy::Slot (&now)[kSegSteps],
+                                            typename Policy::Slot (&next)[kSegSteps], int seg, int next_seg, int ns) {
+    if (pending) cur.commit(rows);
+    pending = cur.room();
+    if (pending) cur.prefetch(rows);
+    pol.load_full(next, next_seg);
+    decode_segment<true, HAS_ESC>(cur, lut, pol, now, seg, ns);
+}
+
+// The walk over one task.  Its first loads (operands of the first segment, the rows that
+// prime the ring) are issued before `between()` runs, which is where the first task of a
+// block copies the decode table into LDS: table, rows and operands are in flight
+// together.  Whole segments alternate between two operand sets (one being decoded, one in
+// flight); the last whole segment reloads itself instead of running past the task.  A
+// last, shorter segment clamps its step indices and guards its steps.
+template <bool HAS_ESC, class Cursor, class Policy, class Between>
+__device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between) {
+    typename Policy::Slot a[kSegSteps], b[kSegSteps];
+    const int full_end = ns - ns % kSegSteps;
+    const int last_full = full_end - kSegSteps;
     pol.prime();
-    cur.prime();
-    cur.start(lut);
-    typename Policy::Slot slot[kSegSteps];
-    uint32_t rows[kSegRows];
-    int seg = 0;
-    for (; seg + kSegSteps <= ns; seg += kSegSteps) {
-        const bool stage = cur.room();
-        if (stage) cur.prefetch(rows);
-        pol.load_full(slot, seg);
-        if (stage) cur.commit(rows);
-        decode_segment<true, HAS_ESC>(cur, lut, pol, slot, seg, ns);
-    }
-    if (seg < ns) {
-        const bool stage = cur.room();
-        if (stage) cur.prefetch(rows);
+    if (full_end > 0) {
+        pol.load_full(a, 0);
+    } else {
 #pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) pol.load(slot[i], seg + i);
-        if (stage) cur.commit(rows);
-        decode_segment<false, HAS_ESC>(cur, lut, pol, slot, seg, ns);
+        for (int i = 0; i < kSegSteps; ++i) pol.load(a[i], i);
     }
+    {
+        uint32_t first[kPrimeRows];
+        cur.prime_issue(first);
+        between();
+        cur.prime_commit(first);
+    }
+    cur.start(lut);
+    uint32_t rows[kSegRows];
+    bool pending = cur.room();
+    if (pending) cur.prefetch(rows);
+    int seg = 0;
+    if (full_end > 0) {
+        for (;;) {
+            int nx = seg + kSegSteps;
+            run_segment<HAS_ESC>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, ns);
+            seg = nx;
+            if (seg >= full_end) break;
+            nx = seg + kSegSteps;
+            run_segment<HAS_ESC>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, ns);
+            seg = nx;
+            if (seg >= full_end) break;
+        }
+        if (seg < ns) {
+#pragma unroll
+            for (int i = 0; i < kSegSteps; ++i) pol.load(a[i], seg + i);
+        }
+    }
+    if (pending) cur.commit(rows);
+    if (seg < ns) decode_segment<false, HAS_ESC>(cur, lut, pol, a, seg, ns);
 }
 
 // The format header (code_lengths buffer): [0] version, [1] table bits, [2] ESC code
@@ -217,8 +252,12 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
                            const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
     __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
-    load_table<Codec::kTableWords>(lut, table);
-    __syncthreads();
+    // The table reaches LDS while the task's first loads are in flight; a wavefront without
+    // a task still copies its share and joins the barrier.
+    auto stage_table = [&]() {
+        load_table<Codec::kTableWords>(lut, table);
+        __syncthreads();
+    };
 
     const int lane = threadIdx.x & (kLanes - 1);
     const int wave = (int)uniform(threadIdx.x / kLanes);
@@ -226,7 +265,10 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
     const int per_group = s.split_k * s.nc;
     const long long ntasks = (long long)G * per_group;
     const long long task = (long long)blockIdx.x * NW + wave;
-    if (task >= ntasks) return;
+    if (task >= ntasks) {
+        stage_table();
+        return;
+    }
     const int g = (int)(task / per_group);
     const TaskId id = task_of(s, (int)(task % per_group));
 
@@ -237,8 +279,8 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
     pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
     pol.yp = Y + (size_t)(kGroupRows * g + (lane & 3)) * K + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols;
     pol.last = id.t1 - id.t0 - 1;
-    if (Codec::variant(header)) run_task<true>(cur, lut, pol, id.t1 - id.t0);
-    else run_task<false>(cur, lut, pol, id.t1 - id.t0);
+    if (Codec::variant(header)) run_task<true>(cur, lut, pol, id.t1 - id.t0, stage_table);
+    else run_task<false>(cur, lut, pol, id.t1 - id.t0, stage_table);
 }
 
 // ------------------------------------------------------------------ fused decode + GEMV
@@ -260,8 +302,17 @@ void gemv_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__
     // The partial sums reuse the rings once every task of the block is done.
     __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
-    load_table<Codec::kTableWords>(lut, table);
-    __syncthreads();
+    // The table reaches LDS while the first task's first loads are in flight: the copy and
+    // its barrier run once per wavefront, inside the first task or, for a wavefront
+    // without one, right after.
+    bool staged = false;
+    auto stage_table = [&]() {
+        if (!staged) {
+            load_table<Codec::kTableWords>(lut, table);
+            __syncthreads();
+            staged = true;
+        }
+    };
 
     const int lane = threadIdx.x & (kLanes - 1);
     const int wave = (int)uniform(threadIdx.x / kLanes);
@@ -292,8 +343,8 @@ void gemv_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__
             }
             pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
-            if (variant) run_task<true>(cur, lut, pol, id.t1 - id.t0);
-            else run_task<false>(cur, lut, pol, id.t1 - id.t0);
+            if (variant) run_task<true>(cur, lut, pol, id.t1 - id.t0, stage_table);
+            else run_task<false>(cur, lut, pol, id.t1 - id.t0, stage_table);
         }
         // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
 #pragma unroll
@@ -308,6 +359,22 @@ void gemv_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__
                 pol.acc[q][i] = a;
             }
         }
+    }
+    stage_table();
+    if (P == 1) {
+        // one wavefront per row group: its sums are final
+        if (active && lane < 4) {
+#pragma unroll
+            for (int q = 0; q < NSET; ++q) {
+                const int batch = lane + 4 * q;
+                if (batch < BS) {
+#pragma unroll
+                    for (int i = 0; i < kGroupRows; ++i)
+                        Y[(size_t)batch * s.M + kGroupRows * g + i] = f32_to_bf16_rne(pol.acc[q][i]);
+                }
+            }
+        }
+        return;
     }
     __syncthreads();                       // every wavefront has finished reading its ring
     float* mine = (float*)rings[wave];     // partial sums: [set][row][batch lane]
