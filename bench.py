@@ -130,6 +130,7 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--algo", default="huffman", choices=["huffman", "ans", "nibble"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-group", action="store_true", help="gate_proj and up_proj as two launches")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1")
@@ -139,6 +140,7 @@ def main():
     from bf16_huffman_infer_amd import _lib
     _lib.load()                                   # fail before any work if the HIP library is missing
     import torch.nn.functional as F
+    from bf16_huffman_infer_amd.functional import linear_grouped
 
     device = torch.device("cuda", 0)
     bs = args.batch
@@ -161,13 +163,24 @@ def main():
 
     state = {"i": 0}
 
-    def step():
+    def step_single():
         mods = blocks[state["i"] % COPIES]
         state["i"] += 1
         for m, x in zip(mods, xs):
             F.linear(x, m)
 
-    sec = time_launches(step, args.steps, args.warmup, launches_per_graph=COPIES)
+    # gate_proj and up_proj multiply the same activations: one grouped launch, as in a
+    # decoder whose projections were tied by cudastream_utils.parallelize_qkv_model
+    def step_grouped():
+        mods = blocks[state["i"] % COPIES]
+        state["i"] += 1
+        F.linear(xs[0], mods[0])
+        F.linear(xs[1], mods[1])
+        linear_grouped(xs[2], [mods[2], mods[3]])
+        F.linear(xs[4], mods[4])
+
+    sec_single = time_launches(step_single, args.steps, args.warmup, launches_per_graph=COPIES)
+    sec = sec_single if args.no_group else time_launches(step_grouped, args.steps, args.warmup, launches_per_graph=COPIES)
     gbs = block_bytes / sec / 1e9
 
     # Per-layer timing and the roofline of the dominant kernel.  A layer alone must not be
@@ -205,7 +218,9 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"Qwen2.5-7B decoder-block linears (qkv 4608x3584, o 3584x3584, gate/up 18944x3584, "
                                f"down 3584x18944), N(0,0.02) seeded, algo={args.algo}, batch={bs}, {COPIES} "
-                               f"alternating weight copies"},
+                               f"alternating weight copies, "
+                               f"{'5 launches' if args.no_group else '4 launches (gate+up grouped)'} per step"},
+        "ms_per_step_single_launches": round(sec_single * 1e3, 5),
         "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "compressed_bytes_per_step": block_bytes, "compression_ratio": round(
             sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),

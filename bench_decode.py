@@ -185,6 +185,7 @@ def main():
     ap.add_argument("--algo", default="smallest", choices=["huffman", "ans", "smallest", "nibble"])
     ap.add_argument("--repeats", type=int, default=3)
     ap.add_argument("--small", action="store_true", help="tiny shapes (smoke run)")
+    ap.add_argument("--no-group", action="store_true", help="q/k/v and gate/up as separate launches")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         sys.exit("bench_decode.py needs a GPU")
@@ -218,6 +219,16 @@ def main():
             kinds[type(m).__name__] = kinds.get(type(m).__name__, 0) + 1
     new_size = get_model_size(model)
     new_ids, new_s = best(model)
+    single_s = None
+    if not args.no_group:
+        # the reference's benchmark runs get_parallelize_qkv_model on the converted model
+        # (examples/benchmark.py:60); here that ties q/k/v and gate/up into grouped launches
+        from bf16_huffman_infer_amd.cudastream_utils import parallelize_qkv_model
+        single_s = new_s
+        del model._graph
+        parallelize_qkv_model(model)
+        grouped_ids, new_s = best(model)
+        assert torch.equal(grouped_ids, new_ids), "grouped launches changed the generated tokens"
     same = int((raw_ids == new_ids).long().cumprod(0).sum().item())
     print(json.dumps({
         "workload": f"Qwen3-8B-shaped decoder ({c.layers} layers, hidden {c.hidden}, intermediate {c.intermediate}, "
@@ -226,6 +237,8 @@ def main():
         "algo": args.algo, "modules": kinds,
         "raw_tokens_per_s": round(args.tokens / raw_s, 2), "compressed_tokens_per_s": round(args.tokens / new_s, 2),
         "compressed_over_raw": round(raw_s / new_s, 4),
+        "launches": "q/k/v and gate/up one launch each" if single_s is not None else "one launch per linear",
+        "compressed_tokens_per_s_single_launches": None if single_s is None else round(args.tokens / single_s, 2),
         "raw_ms_per_token": round(raw_s / args.tokens * 1e3, 4), "compressed_ms_per_token": round(new_s / args.tokens * 1e3, 4),
         "raw_gib": round(raw_size / 2**30, 3), "compressed_gib": round(new_size / 2**30, 3),
         "footprint_ratio": round(new_size / raw_size, 4),

@@ -11,6 +11,16 @@ LIB_PATH = os.path.join(_HERE, "libbhi_hip.so")
 
 _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 
+
+class GemvMember(ctypes.Structure):
+    """``bhi_gemv_member`` of include/bhi.h: one weight of a grouped GEMV launch."""
+    _fields_ = [("A_rem", _vp), ("A_exp", _vp), ("exp_words", _i64), ("Y", _vp), ("offsets", _vp),
+                ("table", _vp), ("table_bytes", _i64), ("header", _vp), ("M", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
+
+
+_grouped = (_i32, [ctypes.POINTER(GemvMember), _i32, _vp, _i32, _i32, _i32, _vp])
+
 _SIGNATURES = {
     "bhi_constants": (_i32, [ctypes.POINTER(ctypes.c_int32), _i32]),
     "bhi_chunks_per_group": (_i32, [_i32, _i32, _i32]),
@@ -29,6 +39,9 @@ _SIGNATURES = {
     "bhi_nibble_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_nibble_encode": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp]),
     "bhi_nibble_encode_capacity": (_i64, [_i32]),
+    "bhi_gemv_bf16_huffman_grouped": _grouped,
+    "bhi_gemv_bf16_ans_grouped": _grouped,
+    "bhi_gemv_bf16_nibble_grouped": _grouped,
     "bhi_reference_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_reference_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
 }

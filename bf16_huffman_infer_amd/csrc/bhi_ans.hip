@@ -113,6 +113,12 @@ extern "C" int bhi_gemv_bf16_ans(const void* A_rem, const void* A_exp, int64_t e
     return bhi_launch_status("gemv_bf16_ans");
 }
 
+extern "C" int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, const void* X,
+                                         int split_k, int Ks, int batch, void* stream) {
+    if (int rc = gemv_grouped<AnsCodec>(members, n_members, X, split_k, Ks, batch, 0, true, (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemv_bf16_ans_grouped");
+}
+
 extern "C" int bhi_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
                               void* Y, const void* offsets, const void* LUT,
                               int split_k, int M, int Ks, void* stream) {

@@ -119,6 +119,13 @@ extern "C" int bhi_gemv_bf16_huffman(const void* A_rem, const void* A_exp, int64
     return bhi_launch_status("gemv_bf16_huffman");
 }
 
+extern "C" int bhi_gemv_bf16_huffman_grouped(const bhi_gemv_member* members, int n_members, const void* X,
+                                             int split_k, int Ks, int batch, void* stream) {
+    if (int rc = gemv_grouped<HuffCodec>(members, n_members, X, split_k, Ks, batch, (int64_t)kTableEntries * 4, false,
+                                         (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemv_bf16_huffman_grouped");
+}
+
 extern "C" int64_t bhi_encode_capacity(int n_steps) {
     if (n_steps < 1) return 0;
     // every lane full of longest codes + every pair escaped + alignment

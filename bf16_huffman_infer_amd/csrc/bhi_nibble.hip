@@ -79,6 +79,12 @@ extern "C" int bhi_gemv_bf16_nibble(const void* A_rem, const void* A_exp, int64_
     return bhi_launch_status("gemv_bf16_nibble");
 }
 
+extern "C" int bhi_gemv_bf16_nibble_grouped(const bhi_gemv_member* members, int n_members, const void* X,
+                                            int split_k, int Ks, int batch, void* stream) {
+    if (int rc = gemv_grouped<NibbleCodec>(members, n_members, X, split_k, Ks, batch, 0, true, (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemv_bf16_nibble_grouped");
+}
+
 extern "C" int bhi_nibble_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
                                  void* Y, const void* offsets, const void* LUT,
                                  int split_k, int M, int Ks, void* stream) {

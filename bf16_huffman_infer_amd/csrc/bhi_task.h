@@ -293,15 +293,47 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
 #endif
 constexpr int min_waves(int bs) { return bs <= 1 ? BHI_MIN_WAVES1 : (bs <= 2 ? 5 : (bs <= 4 ? 4 : 3)); }
 
+// One launch can serve several weights that multiply the same X (the q/k/v or gate/up
+// projections of a decoder layer): each member brings its own buffers, table and output,
+// and owns a contiguous range of the grid.
+constexpr int kMaxMembers = 4;
+struct Member {
+    const uint8_t* rem;
+    const uint32_t* exp;
+    uint16_t* Y;
+    const uint32_t* offsets;
+    const uint32_t* table;
+    const uint8_t* header;
+    Shape s;
+    int first_block;         // this member's blocks are [first_block, next member's first_block)
+};
+struct Group {
+    int n;
+    Member m[kMaxMembers];
+};
+
 template <class Codec, int BS, int NW>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
-void gemv_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
-                         const uint16_t* __restrict__ X, uint16_t* __restrict__ Y,
-                         const uint32_t* __restrict__ offsets, const uint32_t* __restrict__ table,
-                         const uint8_t* __restrict__ header, Shape s, int P, int groups_per_block) {
+void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     // The partial sums reuse the rings once every task of the block is done.
     __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
+    int member = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMembers; ++i)
+        if (i < grp.n && (int)blockIdx.x >= grp.m[i].first_block) member = i;
+    const Member& mb = grp.m[member];
+    const uint8_t* __restrict__ A_rem = mb.rem;
+    const uint32_t* __restrict__ A_exp = mb.exp;
+    uint16_t* __restrict__ Y = mb.Y;
+    const uint32_t* __restrict__ offsets = mb.offsets;
+    const uint32_t* __restrict__ table = mb.table;
+    const uint8_t* __restrict__ header = mb.header;
+    const Shape s = mb.s;
+    const int block = (int)blockIdx.x - mb.first_block;
+    // P wavefronts share one row group; a block holds NW / P row groups
+    const int P = s.split_k * s.nc < NW ? s.split_k * s.nc : NW;
+    const int groups_per_block = NW / P;
     // The table reaches LDS while the first task's first loads are in flight: the copy and
     // its barrier run once per wavefront, inside the first task or, for a wavefront
     // without one, right after.
@@ -319,7 +351,7 @@ void gemv_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__
     const int G = s.M / kGroupRows;
     const int per_group = s.split_k * s.nc;
     const int rg = wave / P, p = wave % P;
-    const int g = blockIdx.x * groups_per_block + rg;
+    const int g = block * groups_per_block + rg;
     const bool active = rg < groups_per_block && g < G;
     const int K = s.Ks * s.split_k;
     const bool variant = Codec::variant(header);
@@ -418,35 +450,75 @@ static inline int check_shape(int split_k, int M, int Ks, int64_t exp_words, bhi
     return 0;
 }
 
-template <class Codec, int BS>
-static inline void launch_gemv(const void* A_rem, const void* A_exp, const void* X, void* Y, const void* offsets,
-                        const void* LUT1, const void* header, const bhi::Shape& s, hipStream_t stream) {
+// Blocks a member needs: one per NW / P row groups.
+static inline int gemv_blocks(const bhi::Shape& s) {
     using namespace bhi;
     const int per_group = s.split_k * s.nc;
-    const int G = s.M / kGroupRows;
-    // P wavefronts share one row group; a block of 8 wavefronts holds 8 / P row groups
-    constexpr int NW = kWavesPerBlock;
-    const int P = per_group < NW ? per_group : NW, gpb = NW / P;
-    hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, NW>), dim3((unsigned)((G + gpb - 1) / gpb)), dim3(NW * kLanes), 0, stream,
-                       (const uint8_t*)A_rem, (const uint32_t*)A_exp, (const uint16_t*)X, (uint16_t*)Y,
-                       (const uint32_t*)offsets, (const uint32_t*)LUT1, (const uint8_t*)header, s, P, gpb);
+    const int P = per_group < kWavesPerBlock ? per_group : kWavesPerBlock, gpb = kWavesPerBlock / P;
+    return (s.M / kGroupRows + gpb - 1) / gpb;
 }
 
+template <class Codec, int BS>
+static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks, hipStream_t stream) {
+    using namespace bhi;
+    hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock>), dim3((unsigned)blocks), dim3(kWavesPerBlock * kLanes),
+                       0, stream, (const uint16_t*)X, grp);
+}
 
+template <class Codec>
+static inline void launch_gemv_batch(int batch, const void* X, const bhi::Group& grp, int blocks, hipStream_t st) {
+    switch (batch) {
+        case 1: launch_gemv<Codec, 1>(X, grp, blocks, st); break;
+        case 2: launch_gemv<Codec, 2>(X, grp, blocks, st); break;
+        case 3: launch_gemv<Codec, 3>(X, grp, blocks, st); break;
+        case 4: launch_gemv<Codec, 4>(X, grp, blocks, st); break;
+        case 5: launch_gemv<Codec, 5>(X, grp, blocks, st); break;
+        case 6: launch_gemv<Codec, 6>(X, grp, blocks, st); break;
+        case 7: launch_gemv<Codec, 7>(X, grp, blocks, st); break;
+        default: launch_gemv<Codec, 8>(X, grp, blocks, st); break;
+    }
+}
+
+// A single weight is a group of one.
 template <class Codec>
 static inline void launch_gemv_batch(int batch, const void* A_rem, const void* A_exp, const void* X, void* Y,
                                      const void* offsets, const void* table, const void* header,
                                      const bhi::Shape& s, hipStream_t st) {
-    switch (batch) {
-        case 1: launch_gemv<Codec, 1>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        case 2: launch_gemv<Codec, 2>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        case 3: launch_gemv<Codec, 3>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        case 4: launch_gemv<Codec, 4>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        case 5: launch_gemv<Codec, 5>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        case 6: launch_gemv<Codec, 6>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        case 7: launch_gemv<Codec, 7>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
-        default: launch_gemv<Codec, 8>(A_rem, A_exp, X, Y, offsets, table, header, s, st); break;
+    bhi::Group grp = {};
+    grp.n = 1;
+    grp.m[0] = bhi::Member{(const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
+                           (const uint32_t*)table, (const uint8_t*)header, s, 0};
+    launch_gemv_batch<Codec>(batch, X, grp, gemv_blocks(s), st);
+}
+
+// The grouped entry points: members of one codec that share X, split_k and Ks.
+// `table_bytes_expected` > 0 checks every member's table size (Huffman).
+template <class Codec>
+static inline int gemv_grouped(const bhi_gemv_member* members, int n_members, const void* X, int split_k, int Ks,
+                               int batch, int64_t table_bytes_expected, bool header_is_table, hipStream_t st) {
+    using namespace bhi;
+    if (!members || !X) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (n_members < 1 || n_members > kMaxMembers) return bhi_fail(BHI_EINVAL, "a group has 1 to 4 members");
+    if (batch < 1) return bhi_fail(BHI_EINVAL, "batch must be >= 1");
+    if (batch > kMaxBatch) return bhi_fail(BHI_EBATCH, "fused GEMV supports batch <= 8");
+    Group grp = {};
+    grp.n = n_members;
+    long long blocks = 0;
+    for (int i = 0; i < n_members; ++i) {
+        const bhi_gemv_member& m = members[i];
+        if (!m.A_rem || !m.A_exp || !m.Y || !m.offsets || !m.table || (!header_is_table && !m.header))
+            return bhi_fail(BHI_EINVAL, "null pointer in a group member");
+        if (table_bytes_expected > 0 && m.table_bytes != table_bytes_expected)
+            return bhi_fail(BHI_ELAYOUT, "decode table of a group member has the wrong size");
+        Shape s;
+        if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &s)) return rc;
+        grp.m[i] = Member{(const uint8_t*)m.A_rem, (const uint32_t*)m.A_exp, (uint16_t*)m.Y, (const uint32_t*)m.offsets,
+                          (const uint32_t*)m.table, (const uint8_t*)(header_is_table ? m.table : m.header), s, (int)blocks};
+        blocks += gemv_blocks(s);
     }
+    if (blocks > 0x7FFFFFFFll) return bhi_fail(BHI_EINVAL, "group too large for one launch");
+    launch_gemv_batch<Codec>(batch, X, grp, (int)blocks, st);
+    return 0;
 }
 
 template <class Codec>

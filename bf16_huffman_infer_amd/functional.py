@@ -19,8 +19,8 @@ from . import _lib
 from .ans import RANSEncoder
 from .huffman import LUTHuffmanEncoder
 from .ops import (ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemv_bf16_ans,
-                  gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode, nibble_decode,
-                  nibble_encode, nibble_encode_capacity)
+                  gemv_bf16_grouped, gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode,
+                  nibble_decode, nibble_encode, nibble_encode_capacity)
 from .utils import get_block_size_n, split_bf16
 
 ANS_PRECISION = 8
@@ -35,6 +35,8 @@ __all__ = [
     "linear_huffman",
     "linear_ans",
     "linear_nibble",
+    "linear_grouped",
+    "LinearGroup",
     "HuffmanWeight",
     "ANSWeight",
     "NibbleWeight",
@@ -348,9 +350,92 @@ class CompressedLinear(nn.Module):
         super().__init__()
         self.weight = weight
         self.bias = bias
+        self._group = None          # a LinearGroup when this module shares launches with siblings
 
     def forward(self, input: Tensor) -> Tensor:
+        group = getattr(self, '_group', None)
+        if group is not None:
+            return group.forward(self, input)
         return F.linear(input, self.weight, self.bias)
+
+
+def linear_grouped(input: Tensor, weights, biases=None) -> list:
+    """``[F.linear(input, w, b) for w, b in zip(weights, biases)]`` in ONE launch.
+
+    ``weights`` are up to four compressed weights of one class with the same
+    ``in_features`` split (``rem.shape[0]`` and ``rem.shape[2]``); ``input`` has at most
+    8 rows after flattening.  This is what the q/k/v (or gate/up) projections of a
+    decoder layer need: the reference overlaps them on parallel streams
+    (``cudastream_utils.py:8-47``), here they are one grid.
+    """
+    assert input.dim() >= 2, input
+    shape = input.shape
+    x = input.flatten(0, -2)
+    if x.size(0) > MAX_FUSED_BATCH:
+        raise RuntimeError(f'linear_grouped takes at most {MAX_FUSED_BATCH} rows, got {x.size(0)}')
+    first = weights[0]
+    split_k, _, N = first.rem.shape
+    x = x.view(-1, split_k, N)
+    _check_weight_call(first.rem, first.exp, x)
+    ys = [torch.empty((x.size(0), w.rem.shape[1]), dtype=torch.bfloat16, device=x.device) for w in weights]
+    gemv_bf16_grouped(weights, x.contiguous(), ys)
+    outs = []
+    for i, y in enumerate(ys):
+        b = None if biases is None else biases[i]
+        if b is not None:
+            y += b[None, :]
+        outs.append(y.unflatten(0, shape[:-1]))
+    return outs
+
+
+class LinearGroup:
+    """Sibling :class:`CompressedLinear` modules that a model always calls one after the
+    other on the same input tensor (q/k/v of an attention block, gate/up of an MLP).
+
+    The call of the first member computes every member's output in one grouped launch
+    and keeps the others until their own call collects them.  Whatever does not fit that
+    pattern -- more than 8 rows, a member called alone or on another tensor, weights of
+    different codecs or splits -- runs each member's ordinary path, so grouping never
+    changes results, only the number of launches.
+    """
+
+    def __init__(self, members):
+        self.members = list(members)
+        for m in self.members:
+            if not isinstance(m, CompressedLinear):
+                raise TypeError('LinearGroup takes CompressedLinear modules')
+        if not 2 <= len(self.members) <= 4:
+            raise ValueError('a group has 2 to 4 members')
+        first = self.members[0].weight
+        self.uniform = all(type(m.weight) is type(first) and m.weight.rem.shape[0] == first.rem.shape[0]
+                           and m.weight.rem.shape[2] == first.rem.shape[2] for m in self.members)
+        self._input = None
+        self._outputs = None
+        for m in self.members:
+            m._group = self
+
+    def dissolve(self) -> None:
+        for m in self.members:
+            m._group = None
+
+    def forward(self, module: CompressedLinear, input: Tensor) -> Tensor:
+        index = next(i for i, m in enumerate(self.members) if m is module)
+        if index == 0:
+            self._input = self._outputs = None
+            rows = input.numel() // input.shape[-1] if input.dim() >= 2 else MAX_FUSED_BATCH + 1
+            if self.uniform and input.is_cuda and rows <= MAX_FUSED_BATCH:
+                self._outputs = linear_grouped(input, [m.weight for m in self.members],
+                                               [m.bias for m in self.members])
+                self._input = input
+                return self._outputs[0]
+        elif self._input is input and self._outputs is not None:
+            out = self._outputs[index]
+            self._outputs[index] = None
+            if index == len(self.members) - 1:
+                self._input = self._outputs = None
+            if out is not None:
+                return out
+        return F.linear(input, module.weight, module.bias)
 
 
 def _weight_bytes(w: nn.Module) -> int:

@@ -269,5 +269,57 @@ def nibble_decode(A_rem: Tensor, A_exp: Tensor, Y: Tensor, offsets: Tensor, LUT:
     torch.ops.bf16_huffman_infer.nibble_decode.default(A_rem, A_exp, Y, offsets, LUT)
 
 
+def gemv_bf16_grouped(weights, X: Tensor, Ys) -> None:
+    """One launch for up to four compressed weights that multiply the same ``X``.
+
+    ``weights`` are weight modules of ONE class (:class:`HuffmanWeight`, :class:`ANSWeight`
+    or :class:`NibbleWeight`: anything with ``rem, exp, offsets`` and ``LUT1, code_lengths``
+    or ``LUT``) with equal ``split_k`` and ``Ks``; ``X`` is bf16 ``[batch, split_k, Ks]``,
+    ``Ys[i]`` bf16 ``[batch, M_i]`` is written.  Not an op of the reference: it stands in
+    for its q/k/v streams (``cudastream_utils.py:8-47``).  Plain function, not registered
+    with the dispatcher; like the ops it only enqueues on the current stream.
+    """
+    if not 1 <= len(weights) <= 4 or len(weights) != len(Ys):
+        raise RuntimeError("a group has 1 to 4 weights and one output per weight")
+    first = weights[0]
+    huffman = hasattr(first, "LUT1")
+    if huffman:
+        entry, name = "bhi_gemv_bf16_huffman_grouped", "gemv_bf16_huffman_grouped"
+    elif int(getattr(first, "MAGIC", 0)) != 0:
+        entry, name = "bhi_gemv_bf16_nibble_grouped", "gemv_bf16_nibble_grouped"
+    else:
+        entry, name = "bhi_gemv_bf16_ans_grouped", "gemv_bf16_ans_grouped"
+    split_k, _, Ks = _weight_dims(first.rem, first.offsets)
+    if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
+        raise RuntimeError(f"X must be [batch, {split_k}, {Ks}], got {tuple(X.shape)}")
+    x_ptr = _req(X, torch.bfloat16, "X", first.rem)
+    batch = X.shape[0]
+    members = (_lib.GemvMember * len(weights))()
+    for m, w, Y in zip(members, weights, Ys):
+        if type(w) is not type(first):
+            raise RuntimeError("the weights of a group must use one codec")
+        sk, M, ks = _weight_dims(w.rem, w.offsets)
+        if (sk, ks) != (split_k, Ks):
+            raise RuntimeError("the weights of a group must share split_k and Ks")
+        if tuple(Y.shape) != (batch, M):
+            raise RuntimeError(f"Y must be [{batch}, {M}], got {tuple(Y.shape)}")
+        m.A_rem = _req(w.rem, torch.uint8, "A_rem", first.rem)
+        m.A_exp = _req(w.exp, torch.int32, "A_exp", first.rem)
+        m.exp_words = w.exp.numel()
+        m.Y = _req(Y, torch.bfloat16, "Y", first.rem)
+        m.offsets = _req(w.offsets, torch.int32, "offsets", first.rem)
+        if huffman:
+            m.table = _req(w.LUT1, torch.uint8, "LUT1", first.rem)
+            m.table_bytes = w.LUT1.numel()
+            m.header = _req(w.code_lengths, torch.uint8, "code_lengths", first.rem)
+        else:
+            m.table = _req(w.LUT, torch.int32, "LUT", first.rem)
+            m.table_bytes = w.LUT.numel() * 4
+            m.header = None
+        m.M = M
+    with torch.cuda.device(first.rem.device):
+        _lib.check(getattr(_lib.load(), entry)(members, len(weights), x_ptr, split_k, Ks, batch, _stream(first.rem)), name)
+
+
 def nibble_encode_capacity(n_steps: int) -> int:
     return int(_lib.load().bhi_nibble_encode_capacity(n_steps))

@@ -127,6 +127,33 @@ int bhi_nibble_encode(const void* data, const void* LUT, void* output, void* out
                       int n_tasks, int n_steps, int64_t out_stride, void* stream);
 int64_t bhi_nibble_encode_capacity(int n_steps);
 
+/* Grouped fused GEMV: up to 4 weights of one codec that multiply the same X (same
+ * split_k and Ks, any M) in ONE launch -- the q/k/v or gate/up projections of a decoder
+ * layer.  Replaces cudastream_utils.py:8-47 of the reference, which runs q/k/v on parallel
+ * streams to the same end (fewer serial launches per token).  Every member is a complete
+ * weight as the single entry points take it, with its own output Y bf16 [batch, M]:
+ *   table/table_bytes  LUT1 + its size (Huffman) or LUT int32[256] (rANS, nibble; size unchecked)
+ *   header             code_lengths (Huffman); ignored for rANS and nibble
+ * `members` is a host array that is read before the call returns. */
+typedef struct bhi_gemv_member {
+    const void* A_rem;
+    const void* A_exp;
+    int64_t exp_words;
+    void* Y;
+    const void* offsets;
+    const void* table;
+    int64_t table_bytes;
+    const void* header;
+    int32_t M;
+    int32_t reserved;
+} bhi_gemv_member;
+int bhi_gemv_bf16_huffman_grouped(const bhi_gemv_member* members, int n_members, const void* X,
+                                  int split_k, int Ks, int batch, void* stream);
+int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, const void* X,
+                              int split_k, int Ks, int batch, void* stream);
+int bhi_gemv_bf16_nibble_grouped(const bhi_gemv_member* members, int n_members, const void* X,
+                                 int split_k, int Ks, int batch, void* stream);
+
 /* Readers for weights that were compressed by the reference package itself: same tensors
  * as the reference's huffman_decode / ans_decode ops (kernel.cu:534-587, 878-919) IN THE
  * REFERENCE'S OWN LAYOUT (functional.py:129-242: 64 streams per row, LUT1..4 uint8 [256],
