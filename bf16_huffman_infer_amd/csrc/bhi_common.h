@@ -108,6 +108,8 @@ constexpr int kSegSteps = BHI_SEG_STEPS;
 #define BHI_RING_ROWS 16
 #endif
 constexpr int kRingRows = BHI_RING_ROWS;
+constexpr int kRingRowsLog2 = kRingRows == 8 ? 3 : kRingRows == 16 ? 4 : kRingRows == 32 ? 5 : -1;
+static_assert(kRingRowsLog2 > 0, "ring of 8, 16 or 32 rows");
 constexpr int kSegRows = BHI_SEG_ROWS;          // rows prefetched per segment
 #ifndef BHI_PRIME_ROWS
 #define BHI_PRIME_ROWS 8
@@ -144,7 +146,11 @@ struct RowRing {
 
     // This lane's word of row p >> 5; the next two rows follow at +kLanes, +2*kLanes words.
     __device__ __forceinline__ const lds_u32* slot_of(uint32_t p) const {
-        return ring + ((p >> 5) & (kRingRows - 1)) * kLanes;
+        // v_bfe_u32 + v_lshl_add_u32; written as shift and mask the compiler makes it three
+        // instructions on the critical path of every step
+        uint32_t slot;
+        asm("v_bfe_u32 %0, %1, 5, %2" : "=v"(slot) : "v"(p), "n"(kRingRowsLog2));
+        return ring + slot * kLanes;
     }
 
     // Stage the first kRingRows rows of the block, once per task, in two halves so that the
@@ -268,6 +274,9 @@ struct HuffCursor : RowRing {
         e[3] = table_entry(tb, w3);
         pos += (t01 + e[2] + e[3]) & 0x3Fu;
         if (HAS_ESC) {
+            // pins the cursor update in front of the branch: the entries then die at it and
+            // the rare path patches them in place, without register copies on the common one
+            asm volatile("" : "+v"(pos));
             const uint32_t any = e[0] | e[1] | e[2] | e[3];
             if (__builtin_expect(ballot((int32_t)any < 0) != 0, 0)) escapes(e);
         }
