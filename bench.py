@@ -30,7 +30,7 @@ STD = 0.02
 # HBM bytes per launch of the dominant kernel (18944x3584), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, each scaled by the same counter's reading for the 256 MiB
 # calibration copy below.  Keyed by (algo, batch); None where it has not been measured.
-MEASURED_TRAFFIC = {("huffman", 1): 94_590_000}
+MEASURED_TRAFFIC = {("huffman", 1): 94_390_000}
 
 
 def make_weight(M, K, seed, device):

@@ -84,3 +84,52 @@ def test_get_graphed_model_on_transformers_qwen3(cuda):
     for _ in range(2):
         got = graphed.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False)
         assert torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_parallelize_qkv_model_on_transformers_qwen3(cuda):
+    """The reference's benchmark recipe, get_graphed_model(get_parallelize_qkv_model(model), cache):
+    transformers' attention and MLP call q/k/v and gate/up one after the other on one tensor, so
+    every layer runs two grouped launches, and generation is unchanged."""
+    from transformers import Qwen3Config, Qwen3ForCausalLM, StaticCache
+    import bf16_huffman_infer_amd.functional as fn
+    from bf16_huffman_infer_amd import convert_all_linear, get_graphed_model
+    from bf16_huffman_infer_amd.cudastream_utils import get_parallelize_qkv_model
+    cfg = Qwen3Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=128, vocab_size=4096, max_position_embeddings=128,
+                      tie_word_embeddings=False)
+    torch.manual_seed(0)
+    model = Qwen3ForCausalLM(cfg).bfloat16().eval()
+    convert_all_linear(model, min_out_features=0, progress=False, algo="huffman")
+    model.cuda()
+    ids = torch.randint(0, 4096, (1, 6), generator=torch.Generator().manual_seed(3)).cuda()
+    want = model.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False)
+    grouped = get_parallelize_qkv_model(model)
+    assert model.model.layers[0].self_attn.q_proj._group is None
+    assert grouped.model.layers[1].mlp.up_proj._group is grouped.model.layers[1].mlp.gate_proj._group is not None
+
+    calls = {"grouped": 0, "single": 0}
+    real_grouped, real_single = fn.gemv_bf16_grouped, fn.gemv_bf16_huffman
+
+    def count_grouped(*a, **k):
+        calls["grouped"] += 1
+        return real_grouped(*a, **k)
+
+    def count_single(*a, **k):
+        calls["single"] += 1
+        return real_single(*a, **k)
+    fn.gemv_bf16_grouped, fn.gemv_bf16_huffman = count_grouped, count_single
+    try:
+        with torch.no_grad():
+            one = grouped(input_ids=ids[:, :1]).logits
+    finally:
+        fn.gemv_bf16_grouped, fn.gemv_bf16_huffman = real_grouped, real_single
+    # per layer: q/k/v and gate/up grouped, o_proj and down_proj alone; lm_head alone
+    assert calls == {"grouped": 2 * cfg.num_hidden_layers, "single": 2 * cfg.num_hidden_layers + 1}
+    with torch.no_grad():
+        assert torch.equal(one, model(input_ids=ids[:, :1]).logits)
+    assert torch.equal(grouped.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False), want)
+    cache = StaticCache(config=cfg, max_cache_len=64)
+    graphed = get_graphed_model(grouped, cache)
+    for _ in range(2):
+        assert torch.equal(graphed.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False), want)
