@@ -27,10 +27,11 @@ LAYERS = [("qkv_proj", 4608, 3584), ("o_proj", 3584, 3584), ("gate_proj", 18944,
 COPIES = 2
 ROTATE_BYTES = 640 << 20
 STD = 0.02
-# HBM bytes per launch of the dominant kernel (18944x3584), from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script, each scaled by the same counter's reading for the 256 MiB
-# calibration copy below.  Keyed by (algo, batch); None where it has not been measured.
-MEASURED_TRAFFIC = {("huffman", 1): 94_390_000}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of this script, each scaled by the same counter's reading for the 256 MiB calibration
+# copy below.  Keyed by (algo, batch, launch): "single" = one 18944x3584 matrix, "group" =
+# gate_proj + up_proj in one launch; None where it has not been measured.
+MEASURED_TRAFFIC = {("huffman", 1, "single"): 94_390_000, ("huffman", 1, "group"): 188_780_000}
 
 
 def make_weight(M, K, seed, device):
@@ -206,9 +207,25 @@ def main():
             st["i"] += 1
         per_layer[name] = time_launches(one, max(100, args.steps), args.warmup, launches_per_graph=len(mods))
         if li == 2:
-            t_dom = per_layer[name]
+            t_single = per_layer[name]
+            # the launch that dominates the step: gate_proj and up_proj as one group, again
+            # rotating over clones (of both) so that no cache level holds the weights
+            ups = rotating(blocks[0][3])[:len(mods)]
+            sg = {"i": 0}
+
+            def pair(sg=sg, mods=mods, ups=ups):
+                i = sg["i"] % len(ups)
+                linear_grouped(xs[2], [mods[i], ups[i]])
+                sg["i"] += 1
+            t_group = time_launches(pair, max(100, args.steps), args.warmup, launches_per_graph=len(ups))
+            del ups
         del mods
-    dom_bytes = gemv_bytes(blocks[0][2], bs, LAYERS[2][1], LAYERS[2][2])
+    single_bytes = gemv_bytes(blocks[0][2], bs, LAYERS[2][1], LAYERS[2][2])
+    group_bytes = single_bytes + gemv_bytes(blocks[0][3], bs, LAYERS[3][1], LAYERS[3][2]) - bs * LAYERS[3][2] * 2  # X once
+    if args.no_group:
+        dom_bytes, t_dom, dom_name = single_bytes, t_single, "18944x3584"
+    else:
+        dom_bytes, t_dom, dom_name = group_bytes, t_group, "group of two 18944x3584 (gate_proj + up_proj)"
     achieved = dom_bytes / t_dom / 1e9
 
     out = {
@@ -229,11 +246,16 @@ def main():
         "bs1_tokens_per_s_28_blocks": round(1.0 / sec / 28, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
         "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{dict(huffman='HuffCodec', ans='AnsCodec', nibble='NibbleCodec')[args.algo]}, {bs}, 4> "
-                               f"18944x3584",
+                               f"{dom_name}",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.algo, bs)),
+                     "traffic": MEASURED_TRAFFIC.get((args.algo, bs, "single" if args.no_group else "group")),
                      "bytes_per_launch": dom_bytes, "us_per_launch": round(t_dom * 1e6, 2)},
+        # the same kernel launched for one 18944x3584 matrix alone
+        "single_launch": {"achieved": round(single_bytes / t_single / 1e9, 1),
+                          "frac": round(single_bytes / t_single / 1e9 / HBM_PEAK_GBS, 4),
+                          "traffic": MEASURED_TRAFFIC.get((args.algo, bs, "single")),
+                          "bytes_per_launch": single_bytes, "us_per_launch": round(t_single * 1e6, 2)},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

@@ -15,7 +15,7 @@ _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 class GemvMember(ctypes.Structure):
     """``bhi_gemv_member`` of include/bhi.h: one weight of a grouped GEMV launch."""
     _fields_ = [("A_rem", _vp), ("A_exp", _vp), ("exp_words", _i64), ("Y", _vp), ("offsets", _vp),
-                ("table", _vp), ("table_bytes", _i64), ("header", _vp), ("M", ctypes.c_int32),
+                ("table", _vp), ("table_bytes", _i64), ("header", _vp), ("bias", _vp), ("M", ctypes.c_int32),
                 ("reserved", ctypes.c_int32)]
 
 

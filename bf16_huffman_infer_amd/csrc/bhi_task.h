@@ -304,6 +304,7 @@ struct Member {
     const uint32_t* offsets;
     const uint32_t* table;
     const uint8_t* header;
+    const uint16_t* bias;    // bf16 [M] or null
     Shape s;
     int first_block;         // this member's blocks are [first_block, next member's first_block)
 };
@@ -311,6 +312,14 @@ struct Group {
     int n;
     Member m[kMaxMembers];
 };
+
+// The sum rounded to BF16; with a bias, that BF16 value plus the bias, rounded again (what a
+// separate BF16 `output += bias` after the product gives).
+__device__ __forceinline__ uint16_t finish_output(float sum, const uint16_t* __restrict__ bias, int row) {
+    uint16_t y = f32_to_bf16_rne(sum);
+    if (bias) y = f32_to_bf16_rne(__uint_as_float((uint32_t)y << 16) + __uint_as_float((uint32_t)bias[row] << 16));
+    return y;
+}
 
 template <class Codec, int BS, int NW>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
@@ -329,6 +338,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     const uint32_t* __restrict__ offsets = mb.offsets;
     const uint32_t* __restrict__ table = mb.table;
     const uint8_t* __restrict__ header = mb.header;
+    const uint16_t* __restrict__ bias = mb.bias;
     const Shape s = mb.s;
     const int block = (int)blockIdx.x - mb.first_block;
     // P wavefronts share one row group; a block holds NW / P row groups
@@ -402,7 +412,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
                 if (batch < BS) {
 #pragma unroll
                     for (int i = 0; i < kGroupRows; ++i)
-                        Y[(size_t)batch * s.M + kGroupRows * g + i] = f32_to_bf16_rne(pol.acc[q][i]);
+                        Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(pol.acc[q][i], bias, kGroupRows * g + i);
                 }
             }
         }
@@ -426,7 +436,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
                 for (int i = 0; i < kGroupRows; ++i) {
                     float a = 0.f;
                     for (int w = 0; w < P; ++w) a += ((const float*)rings[rg * P + w])[(q * kGroupRows + i) * 4 + lane];
-                    Y[(size_t)batch * s.M + kGroupRows * g + i] = f32_to_bf16_rne(a);
+                    Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(a, bias, kGroupRows * g + i);
                 }
             }
         }
@@ -487,7 +497,7 @@ static inline void launch_gemv_batch(int batch, const void* A_rem, const void* A
     bhi::Group grp = {};
     grp.n = 1;
     grp.m[0] = bhi::Member{(const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
-                           (const uint32_t*)table, (const uint8_t*)header, s, 0};
+                           (const uint32_t*)table, (const uint8_t*)header, nullptr, s, 0};
     launch_gemv_batch<Codec>(batch, X, grp, gemv_blocks(s), st);
 }
 
@@ -513,7 +523,8 @@ static inline int gemv_grouped(const bhi_gemv_member* members, int n_members, co
         Shape s;
         if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &s)) return rc;
         grp.m[i] = Member{(const uint8_t*)m.A_rem, (const uint32_t*)m.A_exp, (uint16_t*)m.Y, (const uint32_t*)m.offsets,
-                          (const uint32_t*)m.table, (const uint8_t*)(header_is_table ? m.table : m.header), s, (int)blocks};
+                          (const uint32_t*)m.table, (const uint8_t*)(header_is_table ? m.table : m.header),
+                          (const uint16_t*)m.bias, s, (int)blocks};
         blocks += gemv_blocks(s);
     }
     if (blocks > 0x7FFFFFFFll) return bhi_fail(BHI_EINVAL, "group too large for one launch");

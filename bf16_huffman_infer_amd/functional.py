@@ -378,14 +378,10 @@ def linear_grouped(input: Tensor, weights, biases=None) -> list:
     x = x.view(-1, split_k, N)
     _check_weight_call(first.rem, first.exp, x)
     ys = [torch.empty((x.size(0), w.rem.shape[1]), dtype=torch.bfloat16, device=x.device) for w in weights]
-    gemv_bf16_grouped(weights, x.contiguous(), ys)
-    outs = []
-    for i, y in enumerate(ys):
-        b = None if biases is None else biases[i]
-        if b is not None:
-            y += b[None, :]
-        outs.append(y.unflatten(0, shape[:-1]))
-    return outs
+    if biases is not None:
+        biases = [None if b is None else b.detach().contiguous() for b in biases]
+    gemv_bf16_grouped(weights, x.contiguous(), ys, biases)
+    return [y.unflatten(0, shape[:-1]) for y in ys]
 
 
 class LinearGroup:
@@ -548,6 +544,9 @@ def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tens
     shape = input.shape
     input = input.flatten(0, -2)
     if input.size(0) <= MAX_FUSED_BATCH:
+        if bias is not None and bias.dtype == torch.bfloat16:
+            # the grouped entry point adds the bias in the kernel's last store (same bits, one launch less)
+            return linear_grouped(input, [weight], [bias])[0].unflatten(0, shape[:-1])
         output = fused(input)
         if bias is not None:
             output += bias[None, :]

@@ -269,13 +269,14 @@ def nibble_decode(A_rem: Tensor, A_exp: Tensor, Y: Tensor, offsets: Tensor, LUT:
     torch.ops.bf16_huffman_infer.nibble_decode.default(A_rem, A_exp, Y, offsets, LUT)
 
 
-def gemv_bf16_grouped(weights, X: Tensor, Ys) -> None:
+def gemv_bf16_grouped(weights, X: Tensor, Ys, biases=None) -> None:
     """One launch for up to four compressed weights that multiply the same ``X``.
 
     ``weights`` are weight modules of ONE class (:class:`HuffmanWeight`, :class:`ANSWeight`
     or :class:`NibbleWeight`: anything with ``rem, exp, offsets`` and ``LUT1, code_lengths``
     or ``LUT``) with equal ``split_k`` and ``Ks``; ``X`` is bf16 ``[batch, split_k, Ks]``,
-    ``Ys[i]`` bf16 ``[batch, M_i]`` is written.  Not an op of the reference: it stands in
+    ``Ys[i]`` bf16 ``[batch, M_i]`` is written; ``biases[i]`` (bf16 ``[M_i]`` or None) is added
+    as the reference's separate ``output += bias`` would (``functional.py:403-404``).  Not an op of the reference: it stands in
     for its q/k/v streams (``cudastream_utils.py:8-47``).  Plain function, not registered
     with the dispatcher; like the ops it only enqueues on the current stream.
     """
@@ -295,7 +296,9 @@ def gemv_bf16_grouped(weights, X: Tensor, Ys) -> None:
     x_ptr = _req(X, torch.bfloat16, "X", first.rem)
     batch = X.shape[0]
     members = (_lib.GemvMember * len(weights))()
-    for m, w, Y in zip(members, weights, Ys):
+    if biases is None:
+        biases = [None] * len(weights)
+    for m, w, Y, b in zip(members, weights, Ys, biases):
         if type(w) is not type(first):
             raise RuntimeError("the weights of a group must use one codec")
         sk, M, ks = _weight_dims(w.rem, w.offsets)
@@ -317,6 +320,10 @@ def gemv_bf16_grouped(weights, X: Tensor, Ys) -> None:
             m.table_bytes = w.LUT.numel() * 4
             m.header = None
         m.M = M
+        if b is not None:
+            if tuple(b.shape) != (M,):
+                raise RuntimeError(f"bias must be [{M}], got {tuple(b.shape)}")
+            m.bias = _req(b, torch.bfloat16, "bias", first.rem)
     with torch.cuda.device(first.rem.device):
         _lib.check(getattr(_lib.load(), entry)(members, len(weights), x_ptr, split_k, Ks, batch, _stream(first.rem)), name)
 

@@ -134,6 +134,9 @@ int64_t bhi_nibble_encode_capacity(int n_steps);
  * weight as the single entry points take it, with its own output Y bf16 [batch, M]:
  *   table/table_bytes  LUT1 + its size (Huffman) or LUT int32[256] (rANS, nibble; size unchecked)
  *   header             code_lengths (Huffman); ignored for rANS and nibble
+ *   bias               bf16 [M] or NULL: added to the BF16-rounded product and rounded again,
+ *                      bit for bit the reference's `output += bias` (functional.py:403-404)
+ *                      without its extra launch
  * `members` is a host array that is read before the call returns. */
 typedef struct bhi_gemv_member {
     const void* A_rem;
@@ -144,6 +147,7 @@ typedef struct bhi_gemv_member {
     const void* table;
     int64_t table_bytes;
     const void* header;
+    const void* bias;
     int32_t M;
     int32_t reserved;
 } bhi_gemv_member;

@@ -105,7 +105,8 @@ def test_parallelize_qkv_model_groups_and_matches(cuda):
     x = torch.randn(1, 1, 1024, generator=torch.Generator().manual_seed(9)).bfloat16().cuda()
     want, c0 = _count_launches(lambda: model(x))
     got, c1 = _count_launches(lambda: grouped(x))
-    assert c0 == {"grouped": 0, "single": 5} and c1 == {"grouped": 2, "single": 0}
+    # un-tied: q_proj has a bias and takes the grouped entry point as a group of one
+    assert c0 == {"grouped": 1, "single": 4} and c1 == {"grouped": 2, "single": 0}
     assert torch.equal(got, want)
     # more than 8 rows: every member takes its own decode + GEMM path
     xl = torch.randn(12, 1024, generator=torch.Generator().manual_seed(10)).bfloat16().cuda()
@@ -182,3 +183,18 @@ def test_grouped_rejections(cuda):
     assert lib.bhi_gemv_bf16_huffman_grouped(members, 1, x.data_ptr(), 1, 1024, 1, None) != 0     # null members
     assert b"null pointer" in lib.bhi_last_error_string()
     assert lib.bhi_gemv_bf16_huffman_grouped(None, 1, x.data_ptr(), 1, 1024, 1, None) != 0
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans", "nibble"])
+@pytest.mark.parametrize("bs,M,K", [(1, 256, 1024), (4, 128, 12288), (8, 512, 2048)])
+def test_bias_in_the_kernel_equals_a_separate_bf16_add(cuda, algo, bs, M, K):
+    """The reference adds the bias with a separate BF16 `output += bias` (functional.py:403-404);
+    the kernel's last store must give those bits (K=12288: three splits, summed across wavefronts)."""
+    w = gaussian_weight(M, K, seed=31)
+    mod = _cls(algo).compress(w).cuda()
+    b = (torch.randn(M, generator=torch.Generator().manual_seed(5)) * 0.5).bfloat16().cuda()
+    x = torch.randn(bs, K, generator=torch.Generator().manual_seed(6)).bfloat16().cuda()
+    two_step = torch.nn.functional.linear(x, mod)
+    two_step += b[None, :]
+    fused = torch.nn.functional.linear(x, mod, b)
+    assert torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
