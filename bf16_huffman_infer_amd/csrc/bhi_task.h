@@ -1,8 +1,8 @@
 // Codec-independent part of the kernels: how a task is walked (segments, operand
 // policies), the decode-to-BF16 and fused GEMV kernels, and their launch geometry.  A
-// codec supplies `Cursor` (open / prime / start / prefetch / commit / step), the size of
-// its decode table and `variant(header)`, a wave-uniform choice between two
-// instantiations of the walk.
+// codec supplies `Cursor` (open / prime_issue / prime_commit / start / room / prefetch /
+// commit / step), the size of its decode table and `variant(header)`, a wave-uniform
+// choice between two instantiations of the walk.
 #pragma once
 #include "bhi_common.h"
 #include "bhi_host.h"
