@@ -501,6 +501,8 @@ static inline void launch_gemv_batch(int batch, const void* A_rem, const void* A
     launch_gemv_batch<Codec>(batch, X, grp, gemv_blocks(s), st);
 }
 
+static_assert(sizeof(bhi_gemv_member) == 80, "bindings mirror this struct field by field");
+
 // The grouped entry points: members of one codec that share X, split_k and Ks.
 // `table_bytes_expected` > 0 checks every member's table size (Huffman).
 template <class Codec>

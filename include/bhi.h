@@ -150,7 +150,7 @@ typedef struct bhi_gemv_member {
     const void* bias;
     int32_t M;
     int32_t reserved;
-} bhi_gemv_member;
+} bhi_gemv_member;                 /* 80 bytes: nine 8-byte fields, two ints */
 int bhi_gemv_bf16_huffman_grouped(const bhi_gemv_member* members, int n_members, const void* X,
                                   int split_k, int Ks, int batch, void* stream);
 int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, const void* X,
