@@ -31,11 +31,17 @@ class GraphedCallable:
     returns the static output tensor(s) -- the same storage on every call, so a caller
     that keeps results across calls must clone them.
 
-    No memset is recorded by this class itself; ``fn`` must not allocate-and-zero through
-    paths that record memset nodes (use ``tensor.zero_()``, which is a fill kernel).
+    No memset is recorded by this class itself; ``fn`` must not clear memory through paths
+    that record memset nodes -- ``torch.zeros(...)`` inside a capture is one (build the
+    tensor with an elementwise kernel, or clear a preallocated one with ``tensor.zero_()``).
     """
 
     def __init__(self, fn: Callable, sample_args: Sequence[torch.Tensor], warmup: int = 3):
+        # The graph reads every tensor ``fn`` closes over by ADDRESS.  Holding ``fn`` keeps
+        # those tensors alive for as long as the graph can be replayed; without it they are
+        # freed when the caller's scope ends and the allocator hands their memory to
+        # somebody else while replays still read it.
+        self.fn = fn
         self.static_inputs = [a.clone() for a in sample_args]
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -97,11 +103,16 @@ def apply_graphed(model, cache, replace_generate: bool = True) -> None:
                 return_dict=True,
             ).logits
 
+    zero = torch.zeros((), dtype=dtype, device=device)
+    minus_inf = torch.full((), float("-inf"), dtype=dtype, device=device)
+
     def _step(input_ids, cache_position):
         # the one-token step sees every cache slot up to its own position; an additive
-        # mask over the whole static cache keeps every shape independent of the position
+        # mask over the whole static cache keeps every shape independent of the position.
+        # One elementwise kernel from two constants: nothing is zero-filled inside the
+        # capture, so no memset node is recorded.
         visible = key_index[None, None, None, :] <= cache_position.view(1, 1, 1, 1)
-        mask = torch.zeros(1, 1, 1, max_len, dtype=dtype, device=device).masked_fill_(~visible, float("-inf"))
+        mask = torch.where(visible, zero, minus_inf)
         return _forward(input_ids, mask, cache_position.view(1, 1), cache_position)
 
     # recorded at the last cache slot so that the warm-up runs do not disturb a prompt

@@ -79,11 +79,46 @@ def test_get_graphed_model_on_transformers_qwen3(cuda):
     assert any(type(m).__name__ == "HuffmanWeight" for m in model.modules())
     ids = torch.randint(0, 4096, (1, 6), generator=torch.Generator().manual_seed(3)).cuda()
     want = model.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False)
-    cache = StaticCache(config=cfg, max_cache_len=64)
+    cache = StaticCache(config=cfg, max_cache_len=1024)
     graphed = get_graphed_model(model, cache)
-    for _ in range(2):
+    for _ in range(3):
         got = graphed.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False)
         assert torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_graphed_step_replays_are_identical_and_match_eager_on_transformers_qwen3(cuda):
+    """Same tokens from the same cache state: every replay of the recorded step gives the
+    same logits bit for bit (first replay included), and they agree with the model's own
+    eager one-token forward over a static cache of the same length."""
+    from transformers import Qwen3Config, Qwen3ForCausalLM, StaticCache
+    from bf16_huffman_infer_amd import get_graphed_model
+    cfg = Qwen3Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8,
+                      num_key_value_heads=2, head_dim=128, vocab_size=4096, max_position_embeddings=2048,
+                      tie_word_embeddings=False)
+    torch.manual_seed(1)
+    model = Qwen3ForCausalLM(cfg).bfloat16().eval().cuda()
+    ids = torch.randint(0, 4096, (1, 16), generator=torch.Generator().manual_seed(3)).cuda()
+    toks = [7, 99, 1234, 4000]
+
+    def run(m, cache):
+        cache.reset()
+        outs = []
+        with torch.no_grad():
+            outs.append(m(input_ids=ids, past_key_values=cache, use_cache=True).logits[0, -1].float().clone())
+            for t in toks:
+                tok = torch.full((1, 1), t, device="cuda")
+                outs.append(m(input_ids=tok, past_key_values=cache, use_cache=True).logits[0, -1].float().clone())
+        return outs
+
+    eager = run(model, StaticCache(config=cfg, max_cache_len=1024))
+    cache = StaticCache(config=cfg, max_cache_len=1024)
+    graphed = get_graphed_model(model, cache)
+    runs = [run(graphed, cache) for _ in range(3)]
+    for r in runs[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(runs[0], r))
+    for a, b in zip(runs[0], eager):
+        torch.testing.assert_close(a, b, rtol=0, atol=0.08)
 
 
 @pytest.mark.gpu
@@ -129,7 +164,31 @@ def test_parallelize_qkv_model_on_transformers_qwen3(cuda):
     with torch.no_grad():
         assert torch.equal(one, model(input_ids=ids[:, :1]).logits)
     assert torch.equal(grouped.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False), want)
-    cache = StaticCache(config=cfg, max_cache_len=64)
+    cache = StaticCache(config=cfg, max_cache_len=1024)
     graphed = get_graphed_model(grouped, cache)
     for _ in range(2):
         assert torch.equal(graphed.generate(ids, max_new_tokens=12, min_new_tokens=12, do_sample=False), want)
+
+
+@pytest.mark.gpu
+def test_graphed_callable_keeps_closed_over_tensors_alive(cuda):
+    """A recorded function reads the tensors it closes over by address; the callable must keep
+    them alive after the scope that built it is gone (they used to be freed and their memory
+    reused, and replays read whatever landed there)."""
+    import gc
+    from bf16_huffman_infer_amd.cudagraph_utils import GraphedCallable
+
+    def make():
+        table = torch.arange(1024, device="cuda", dtype=torch.float32)
+
+        def fn(x):
+            return x + table
+        return GraphedCallable(fn, (torch.zeros(1024, device="cuda"),))
+
+    step = make()
+    gc.collect()
+    junk = [torch.full((1024,), 7.0, device="cuda") for _ in range(256)]      # same size class as the table
+    out = step(torch.ones(1024, device="cuda"))
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.arange(1024, device="cuda", dtype=torch.float32) + 1)
+    del junk
