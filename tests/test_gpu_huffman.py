@@ -145,3 +145,31 @@ def test_long_incompressible_tasks_outrun_the_row_ring(cuda, algo):
     y = torch.nn.functional.linear(x, mod)
     ref = x.float() @ w.cuda().float().T
     torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans", "nibble"])
+def test_hip_encoders_reproduce_the_format_digests(cuda, algo):
+    """HIP-compressed buffers of the seeded matrices hash to the committed digests of the
+    stream format (tests/golden/wave64_digests.json, written by the numpy model)."""
+    import hashlib
+    import importlib.util
+    import json
+    import os
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight, NibbleWeight
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_wave64_digests", os.path.join(here, "make_wave64_digests.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    want = json.load(open(os.path.join(here, "wave64_digests.json")))
+    sha = lambda t: hashlib.sha256(t.contiguous().cpu().numpy().tobytes()).hexdigest()
+    cls = {"huffman": HuffmanWeight, "ans": ANSWeight, "nibble": NibbleWeight}[algo]
+    for kind, M, K, split_k, seed in gen.CASES:
+        w = MAKERS[kind](M, K, seed=seed)
+        mod = cls.compress_split_n(w, n=split_k)
+        ref = want[f"{kind}_{M}x{K}_split{split_k}_seed{seed}"][algo]
+        assert mod.exp.numel() == ref["exp_words"]
+        assert (sha(mod.rem), sha(mod.exp), sha(mod.offsets)) == (ref["rem"], ref["exp"], ref["offsets"])
+        if algo == "huffman":
+            assert sha(mod.LUT1) == ref["table"]
+        elif algo == "nibble":
+            assert str(int(mod.LUT[0])) == ref["table"]
