@@ -146,11 +146,34 @@ class HuffmanWeight(nn.Module):
         """One code per weight matrix, built from the histogram of exponent pairs."""
         device = torch.device('cuda', 0)
         _, exp = split_bf16(a.detach().to(device))
-        pairs = exp[:, 0::2].to(torch.int32) | (exp[:, 1::2].to(torch.int32) << 8)
-        counts = torch.bincount(pairs.flatten(), minlength=65536)
+        counts = cls._pair_counts(exp)
         codec = LUTHuffmanEncoder()
         codec.build_lut(counts.cpu())
         return codec
+
+    @staticmethod
+    def _pair_counts(exp: Tensor) -> Tensor:
+        """int64 [65536]: occurrences of every exponent pair ``a | b << 8`` (a = even column).
+
+        A histogram over 65536 bins runs on global atomics (25 ms for a 4096x12288 layer); real
+        weights use a few dozen exponent values, so the pairs are counted over the ranks of
+        the values that occur (at most 64 x 64 bins, which the histogram kernel keeps in
+        shared memory) and scattered back."""
+        single = torch.bincount(exp.flatten().to(torch.int32), minlength=256)
+        present = torch.nonzero(single).flatten()                      # exponent values that occur, ascending
+        a, b = exp[:, 0::2], exp[:, 1::2]
+        if present.numel() > 64:
+            pairs = a.to(torch.int32) | (b.to(torch.int32) << 8)
+            return torch.bincount(pairs.flatten(), minlength=65536)
+        rank = torch.zeros(256, dtype=torch.int32, device=exp.device)
+        rank[present] = torch.arange(present.numel(), dtype=torch.int32, device=exp.device)
+        dense = rank[a.to(torch.int64)] | (rank[b.to(torch.int64)] << 6)
+        small = torch.bincount(dense.flatten(), minlength=4096)        # [rank_b * 64 + rank_a]
+        counts = torch.zeros(65536, dtype=torch.int64, device=exp.device)
+        ra, rb = torch.meshgrid(torch.arange(present.numel(), device=exp.device),
+                                torch.arange(present.numel(), device=exp.device), indexing='ij')
+        counts[(present[ra] | (present[rb] << 8)).flatten()] = small[(ra | (rb << 6)).flatten()]
+        return counts
 
     @classmethod
     def get_lut_kwargs(cls, codec: LUTHuffmanEncoder) -> dict[str, Tensor]:

@@ -173,3 +173,15 @@ def test_hip_encoders_reproduce_the_format_digests(cuda, algo):
             assert sha(mod.LUT1) == ref["table"]
         elif algo == "nibble":
             assert str(int(mod.LUT[0])) == ref["table"]
+
+
+@pytest.mark.parametrize("kind", ["gauss", "t3", "bits", "special", "zeros"])
+def test_pair_histogram_shortcut_equals_the_full_histogram(cuda, kind):
+    """The rank-compressed pair histogram of the converter equals a plain 65536-bin count."""
+    from bf16_huffman_infer_amd.functional import HuffmanWeight
+    from bf16_huffman_infer_amd.utils import split_bf16
+    w = MAKERS[kind](256, 1024, seed=9)
+    _, exp = split_bf16(w.cuda())
+    got = HuffmanWeight._pair_counts(exp)
+    assert got.dtype == torch.int64 and got.shape == (65536,)
+    assert np.array_equal(got.cpu().numpy(), pair_counts(bits_of(w)))
