@@ -566,6 +566,8 @@ def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tens
     assert input.dim() >= 2, input
     shape = input.shape
     input = input.flatten(0, -2)
+    if input.size(0) == 0:                       # no rows: nothing to launch
+        return input.new_empty((*shape[:-1], weight.rem.shape[1]))
     if input.size(0) <= MAX_FUSED_BATCH:
         if bias is not None and bias.dtype == torch.bfloat16:
             # the grouped entry point adds the bias in the kernel's last store (same bits, one launch less)

@@ -185,3 +185,12 @@ def test_pair_histogram_shortcut_equals_the_full_histogram(cuda, kind):
     got = HuffmanWeight._pair_counts(exp)
     assert got.dtype == torch.int64 and got.shape == (65536,)
     assert np.array_equal(got.cpu().numpy(), pair_counts(bits_of(w)))
+
+
+def test_linear_with_no_rows(cuda):
+    """An input without rows gives an output without rows (and launches nothing)."""
+    mod = _compress(gaussian_weight(128, 1024, seed=1)).cuda()
+    y = torch.nn.functional.linear(torch.empty(0, 1024, dtype=torch.bfloat16, device="cuda"), mod)
+    assert y.shape == (0, 128) and y.dtype == torch.bfloat16
+    y = torch.nn.functional.linear(torch.empty(2, 0, 1024, dtype=torch.bfloat16, device="cuda"), mod)
+    assert y.shape == (2, 0, 128)
