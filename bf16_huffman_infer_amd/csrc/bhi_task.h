@@ -131,12 +131,12 @@ struct StorePolicy {
     __device__ __forceinline__ void prime() const {}
     __device__ __forceinline__ void load(Slot& s, int t) const {
         t = t < last ? t : last;
-        s.rem = rem0[(size_t)t * kLanes];
+        s.rem = stream_load(rem0 + (size_t)t * kLanes);
     }
     __device__ __forceinline__ void load_full(Slot (&s)[kSegSteps], int t0) const {
         const uint2* p = rem0 + (size_t)t0 * kLanes;
 #pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) s[i].rem = p[i * kLanes];
+        for (int i = 0; i < kSegSteps; ++i) s[i].rem = stream_load(p + i * kLanes);
     }
     __device__ __forceinline__ Piped take(const Slot&, int, int) const { return Piped{}; }
     __device__ __forceinline__ void use(const Piped&, int t, const uint32_t (&w)[4]) const {
@@ -192,7 +192,7 @@ struct MfmaPolicy {
     }
     __device__ __forceinline__ void load(Slot& s, int t) const {
         t = t < last ? t : last;
-        s.rem = rem0[(size_t)t * kLanes];
+        s.rem = stream_load(rem0 + (size_t)t * kLanes);
         if (QUARTER) s.x.x = xq0[(size_t)t * (kStepCols / 2)];
         else if (!PIPED) s.x = x0[0][(size_t)t * (kStepCols / 8)];
     }
@@ -202,7 +202,7 @@ struct MfmaPolicy {
         const uint4* px = x0[0] + (size_t)t0 * (kStepCols / 8);
 #pragma unroll
         for (int i = 0; i < kSegSteps; ++i) {
-            s[i].rem = pr[i * kLanes];
+            s[i].rem = stream_load(pr + i * kLanes);
             if (QUARTER) s[i].x.x = pq[i * (kStepCols / 2)];
             else if (!PIPED) s[i].x = px[i * (kStepCols / 8)];
         }
