@@ -23,6 +23,7 @@ ESC_FLAG = 1 << 31
 ESC_INDEX = 65536
 ESC_SIDE_BITS = 32            # one stream word per escaped pair
 MAX_CODED = 1536              # never give more than this many pairs a code of their own
+ESC_FREE_SHIFT = 5            # an escape-free code may be 1/32 longer than the shortest one
 
 
 def package_merge(weights, max_len: int):
@@ -127,16 +128,25 @@ class LUTHuffmanEncoder:
         present = np.nonzero(counts)[0]
         present = present[np.argsort(-counts[present], kind='stable')]      # most frequent first
         # candidate cut-offs: everything, or only pairs seen at least 2/4/16 times
-        best = None
+        best = free = last = None
         for thr in (1, 2, 4, 16):
             coded = present[counts[present] >= thr][:MAX_CODED]
             if len(coded) == 0:
                 coded = present[:1]
-            if best is not None and len(coded) == len(best[0]):
+            if last is not None and len(coded) == last:
                 continue
+            last = len(coded)
             lengths, bits = self._lengths_for(counts, coded)
+            if len(coded) == len(present):
+                free = (coded, lengths, bits)           # every pair has a code: nothing escapes
             if best is None or bits < best[2]:
                 best = (coded, lengths, bits)
+        # A matrix whose header says "no escapes" is decoded by kernels without the escape
+        # test: one test and one branch less in every step, 6-9 % of a fused GEMV.  Rare
+        # pairs crowd the 11-bit code space, so the escape-free code is a little longer
+        # (2 % on Gaussian weights); it is taken unless it costs more than 1/32.
+        if free is not None and free[2] <= best[2] + (best[2] >> ESC_FREE_SHIFT):
+            best = free
         coded, lengths, self.expected_bits = best
 
         # canonical assignment: shorter codes first, ties by pair id, ESC last in its class
