@@ -150,20 +150,39 @@ __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, Q * 0x55, 0xF, 0xF, true);
 }
 
-// fused GEMV on the matrix cores: v_mfma_f32_4x4x4_16b_bf16 multiplies, in each of its
-// 16 blocks, 4 rows x 4 k (operand A: lane 4*blk + row holds the 4 k values of that row)
-// by 4 k x 4 columns (operand B: lane 4*blk + col) into D[row][col] (register `row` of lane
-// 4*blk + col).  A lane's four pairs are exactly two A operands (columns 0..3 and 4..7 of
-// its row); lane 4*b + j supplies X[batch j] for those columns.  One accumulator set
+// fused GEMV, batch 2..8, on the matrix cores: v_mfma_f32_4x4x4_16b_bf16 multiplies, in each
+// of its 16 blocks, 4 rows x 4 k (operand A: lane 4*blk + row holds the 4 k values of that
+// row) by 4 k x 4 columns (operand B: lane 4*blk + col) into D[row][col] (register `row` of
+// lane 4*blk + col).  A lane's four pairs are exactly two A operands (columns 0..3 and 4..7
+// of its row); lane 4*b + j supplies X[batch j] for those columns.  One accumulator set
 // covers batches 0..3, a second one batches 4..7.  Lanes whose batch does not exist
 // carry finite filler and their results are never stored.
 //
-// How X reaches the B operand depends on the batch:
+// Batch 1 has one column of X: three quarters of such a product would be filler.  There a
+// lane keeps its own row's sum and adds four two-element dot products per step
+// (v_dot2c_f32_bf16, fp32 accumulation like the matrix cores).
+//
+// How X reaches the arithmetic depends on the batch:
 //   batch 1     the four lanes of a quad own the same 8 columns; each loads one X pair
-//               in the load phase (one register per step) and the quad shares them by DPP;
+//               in the load phase (one register per step) and the dot products read the
+//               other lanes' pairs through their DPP operand;
 //   batch 2..4  every lane loads its batch's 8 columns in the load phase (4 registers/step);
 //   batch 5..8  two sets would need 8 registers per step: X is fetched two steps ahead
 //               inside the compute phase instead (it is cache resident).
+//
+// acc += x[q].lo * w.lo + x[q].hi * w.hi, where x[q] is the X pair held by lane q of this
+// lane's quad: v_dot2c_f32_bf16 with the quad broadcast folded into its DPP operand (the
+// compiler keeps a separate v_mov_dpp when given the builtins).  `x` must come straight
+// from a load: a VALU write to it right before a DPP read would need two wait states.
+template <int Q>
+__device__ __forceinline__ void dot_quad(float& acc, uint32_t x, uint32_t w) {
+    static_assert(Q >= 0 && Q < 4, "a quad has four lanes");
+    if (Q == 0) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
+    if (Q == 1) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
+    if (Q == 2) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
+    if (Q == 3) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
+}
+
 template <int BS>
 struct MfmaPolicy {
     static constexpr int NSET = BS <= 4 ? 1 : 2;
@@ -178,6 +197,7 @@ struct MfmaPolicy {
     int last;
     uint4 xr[XAHEAD][NSET];
     f32x4_t acc[NSET];
+    float dot;               // batch 1: this lane's row over its 8 columns of every step so far
 
     __device__ __forceinline__ void xload(uint4 (&dst)[NSET], int t) const {
         t = t < last ? t : last;
@@ -210,7 +230,7 @@ struct MfmaPolicy {
     __device__ __forceinline__ Piped take(const Slot& s, int i, int t) {
         Piped p;
         if (QUARTER) {
-            p.x[0] = make_uint4(s.x.x, quad_bcast<1>(s.x.x), quad_bcast<2>(s.x.x), quad_bcast<3>(s.x.x));
+            p.x[0].x = s.x.x;
         } else if (!PIPED) {
             p.x[0] = s.x;
         } else {
@@ -221,6 +241,13 @@ struct MfmaPolicy {
         return p;
     }
     __device__ __forceinline__ void use(const Piped& s, int, const uint32_t (&w)[4]) {
+        if (QUARTER) {
+            dot_quad<0>(dot, s.x[0].x, w[0]);
+            dot_quad<1>(dot, s.x[0].x, w[1]);
+            dot_quad<2>(dot, s.x[0].x, w[2]);
+            dot_quad<3>(dot, s.x[0].x, w[3]);
+            return;
+        }
         const bf16x4_t a01 = __builtin_bit_cast(bf16x4_t, make_uint2(w[0], w[1]));
         const bf16x4_t a23 = __builtin_bit_cast(bf16x4_t, make_uint2(w[2], w[3]));
 #pragma unroll
@@ -229,6 +256,15 @@ struct MfmaPolicy {
             const bf16x4_t b23 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].z, s.x[q].w));
             acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a01, b01, acc[q], 0, 0, 0);
             acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a23, b23, acc[q], 0, 0, 0);
+        }
+    }
+    // Batch 1 keeps one sum per lane (row lane & 3, column block lane >> 2); hand it over in the
+    // accumulator layout of the matrix cores: register i of a quad's lanes = the sum of row i.
+    __device__ __forceinline__ void fold() {
+        if (QUARTER) {
+            const uint32_t d = __float_as_uint(dot);
+            acc[0] = f32x4_t{__uint_as_float(quad_bcast<0>(d)), __uint_as_float(quad_bcast<1>(d)),
+                             __uint_as_float(quad_bcast<2>(d)), __uint_as_float(quad_bcast<3>(d))};
         }
     }
 };
@@ -370,6 +406,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     constexpr int NSET = MfmaPolicy<BS>::NSET;
 #pragma unroll
     for (int q = 0; q < NSET; ++q) pol.acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    pol.dot = 0.f;
 
     if (active) {
         for (int kc = p; kc < per_group; kc += P) {
@@ -388,6 +425,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
             if (variant) run_task<true>(cur, lut, pol, id.t1 - id.t0, stage_table);
             else run_task<false>(cur, lut, pol, id.t1 - id.t0, stage_table);
         }
+        pol.fold();
         // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
 #pragma unroll
         for (int q = 0; q < NSET; ++q) {
