@@ -9,7 +9,6 @@
 
 namespace bhi {
 
-typedef short bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // Cooperative copy of the decode table into LDS.
@@ -150,25 +149,23 @@ __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, Q * 0x55, 0xF, 0xF, true);
 }
 
-// fused GEMV, batch 2..8, on the matrix cores: v_mfma_f32_4x4x4_16b_bf16 multiplies, in each
-// of its 16 blocks, 4 rows x 4 k (operand A: lane 4*blk + row holds the 4 k values of that
-// row) by 4 k x 4 columns (operand B: lane 4*blk + col) into D[row][col] (register `row` of
-// lane 4*blk + col).  A lane's four pairs are exactly two A operands (columns 0..3 and 4..7
-// of its row); lane 4*b + j supplies X[batch j] for those columns.  One accumulator set
-// covers batches 0..3, a second one batches 4..7.  Lanes whose batch does not exist
-// carry finite filler and their results are never stored.
+// fused GEMV, batch 1..8: a lane keeps the sums of its own row (lane & 3) over its 8 columns
+// of every step, one fp32 accumulator per batch row, and adds four two-element dot
+// products per step and batch row (v_dot2c_f32_bf16).  The four lanes of a quad own the
+// same 8 columns: each loads ONE X pair per batch row (lane 4*b + i the pair 8*b + 2*i,
+// 8*b + 2*i + 1), so a wavefront's X load is 256 contiguous bytes per batch row, and the
+// dot products read the other lanes' pairs through their DPP operand.
 //
-// Batch 1 has one column of X: three quarters of such a product would be filler.  There a
-// lane keeps its own row's sum and adds four two-element dot products per step
-// (v_dot2c_f32_bf16, fp32 accumulation like the matrix cores).
+// (The 4x4x4 matrix products this replaced need, in lane 4*b + j, all 8 columns of batch
+// row j: four different rows of X inside every quad.  Those loads are not coalesced and
+// cost more than everything else the batch adds: 27.9 -> 24.0 us at batch 2, 33.1 -> 27.2
+// at batch 4, 44.6 -> 33.4 at batch 8 on 18944x3584.)
 //
-// How X reaches the arithmetic depends on the batch:
-//   batch 1     the four lanes of a quad own the same 8 columns; each loads one X pair
-//               in the load phase (one register per step) and the dot products read the
-//               other lanes' pairs through their DPP operand;
-//   batch 2..4  every lane loads its batch's 8 columns in the load phase (4 registers/step);
-//   batch 5..8  two sets would need 8 registers per step: X is fetched two steps ahead
-//               inside the compute phase instead (it is cache resident).
+// Where the X pairs wait for their step depends on the batch:
+//   batch 1..4  in the segment's operand set, loaded a segment ahead like rem (bs registers
+//               per step);
+//   batch 5..8  that would be 8 * bs registers: they are fetched XAHEAD steps ahead instead,
+//               right after the step that used their registers (X is cache resident).
 //
 // acc += x[q].lo * w.lo + x[q].hi * w.hi, where x[q] is the X pair held by lane q of this
 // lane's quad: v_dot2c_f32_bf16 with the quad broadcast folded into its DPP operand (the
@@ -184,25 +181,32 @@ __device__ __forceinline__ void dot_quad(float& acc, uint32_t x, uint32_t w) {
 }
 
 template <int BS>
-struct MfmaPolicy {
-    static constexpr int NSET = BS <= 4 ? 1 : 2;
-    static constexpr bool QUARTER = BS == 1;
+struct DotPolicy {
+    static constexpr int NSET = BS <= 4 ? 1 : 2;            // batch rows in sets of four
     static constexpr bool PIPED = BS > 4;
-    static constexpr int XAHEAD = 2;
-    struct Slot { uint2 rem; uint4 x; };         // x: full columns (batch 2..4) or .x = own pair (batch 1)
-    struct Piped { uint4 x[NSET]; };
+    static constexpr int XAHEAD = BS > 6 ? 1 : 2;            // 92 registers at batch 8: five wavefronts per SIMD
+    struct Slot { uint2 rem; uint4 x; };                     // x: the lane's X pair of batch rows 0..3
+    struct Piped { uint4 x; int i, t; };
     const uint2* rem0;
-    const uint4* x0[NSET];   // this lane's 8 X columns of the task's first step, per set
-    const uint32_t* xq0;     // batch 1: this lane's own X pair of the task's first step
+    const uint32_t* xq0;     // this lane's X pair of batch row 0, first step of the task
+    int xrow;                // distance between batch rows of X, in pairs
     int last;
-    uint4 xr[XAHEAD][NSET];
-    f32x4_t acc[NSET];
-    float dot;               // batch 1: this lane's row over its 8 columns of every step so far
+    uint4 xr[XAHEAD][NSET];  // batch 5..8: the pairs of the next XAHEAD steps
+    float dot[2 * 4];
+    f32x4_t acc[NSET];       // filled by fold(): the sums in the layout the epilogue stores from
 
+    // one X pair per batch row B0 .. B0 + 3: each a 256-byte contiguous load of the wavefront
+    template <int B0>
+    __device__ __forceinline__ void xpairs(uint4& x, const uint32_t* p) const {
+        if (BS > B0) x.x = p[(size_t)B0 * xrow];
+        if (BS > B0 + 1) x.y = p[(size_t)(B0 + 1) * xrow];
+        if (BS > B0 + 2) x.z = p[(size_t)(B0 + 2) * xrow];
+        if (BS > B0 + 3) x.w = p[(size_t)(B0 + 3) * xrow];
+    }
     __device__ __forceinline__ void xload(uint4 (&dst)[NSET], int t) const {
         t = t < last ? t : last;
-#pragma unroll
-        for (int q = 0; q < NSET; ++q) dst[q] = x0[q][(size_t)t * (kStepCols / 8)];
+        xpairs<0>(dst[0], xq0 + (size_t)t * (kStepCols / 2));
+        if (NSET > 1) xpairs<4>(dst[NSET - 1], xq0 + (size_t)t * (kStepCols / 2));
     }
     __device__ __forceinline__ void prime() {
         if (PIPED) {
@@ -213,58 +217,58 @@ struct MfmaPolicy {
     __device__ __forceinline__ void load(Slot& s, int t) const {
         t = t < last ? t : last;
         s.rem = stream_load(rem0 + (size_t)t * kLanes);
-        if (QUARTER) s.x.x = xq0[(size_t)t * (kStepCols / 2)];
-        else if (!PIPED) s.x = x0[0][(size_t)t * (kStepCols / 8)];
+        if (!PIPED) xpairs<0>(s.x, xq0 + (size_t)t * (kStepCols / 2));
     }
     __device__ __forceinline__ void load_full(Slot (&s)[kSegSteps], int t0) const {
         const uint2* pr = rem0 + (size_t)t0 * kLanes;
         const uint32_t* pq = xq0 + (size_t)t0 * (kStepCols / 2);
-        const uint4* px = x0[0] + (size_t)t0 * (kStepCols / 8);
 #pragma unroll
         for (int i = 0; i < kSegSteps; ++i) {
             s[i].rem = stream_load(pr + i * kLanes);
-            if (QUARTER) s[i].x.x = pq[i * (kStepCols / 2)];
-            else if (!PIPED) s[i].x = px[i * (kStepCols / 8)];
+            if (!PIPED) xpairs<0>(s[i].x, pq + i * (kStepCols / 2));
         }
     }
-    __device__ __forceinline__ Piped take(const Slot& s, int i, int t) {
+    __device__ __forceinline__ Piped take(const Slot& s, int i, int t) const {
         Piped p;
-        if (QUARTER) {
-            p.x[0].x = s.x.x;
-        } else if (!PIPED) {
-            p.x[0] = s.x;
-        } else {
-#pragma unroll
-            for (int q = 0; q < NSET; ++q) p.x[q] = xr[i % XAHEAD][q];
-            xload(xr[i % XAHEAD], t + XAHEAD);
-        }
+        if (!PIPED) p.x = s.x;
+        p.i = i;
+        p.t = t;
         return p;
     }
     __device__ __forceinline__ void use(const Piped& s, int, const uint32_t (&w)[4]) {
-        if (QUARTER) {
-            dot_quad<0>(dot, s.x[0].x, w[0]);
-            dot_quad<1>(dot, s.x[0].x, w[1]);
-            dot_quad<2>(dot, s.x[0].x, w[2]);
-            dot_quad<3>(dot, s.x[0].x, w[3]);
-            return;
-        }
-        const bf16x4_t a01 = __builtin_bit_cast(bf16x4_t, make_uint2(w[0], w[1]));
-        const bf16x4_t a23 = __builtin_bit_cast(bf16x4_t, make_uint2(w[2], w[3]));
 #pragma unroll
         for (int q = 0; q < NSET; ++q) {
-            const bf16x4_t b01 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].x, s.x[q].y));
-            const bf16x4_t b23 = __builtin_bit_cast(bf16x4_t, make_uint2(s.x[q].z, s.x[q].w));
-            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a01, b01, acc[q], 0, 0, 0);
-            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a23, b23, acc[q], 0, 0, 0);
+            const uint4 xs = PIPED ? xr[s.i % XAHEAD][q] : s.x;
+            const uint32_t xb[4] = {xs.x, xs.y, xs.z, xs.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (4 * q + j < BS) {
+                    dot_quad<0>(dot[4 * q + j], xb[j], w[0]);
+                    dot_quad<1>(dot[4 * q + j], xb[j], w[1]);
+                    dot_quad<2>(dot[4 * q + j], xb[j], w[2]);
+                    dot_quad<3>(dot[4 * q + j], xb[j], w[3]);
+                }
+            }
         }
+        if (PIPED) xload(xr[s.i % XAHEAD], s.t + XAHEAD);
     }
-    // Batch 1 keeps one sum per lane (row lane & 3, column block lane >> 2); hand it over in the
-    // accumulator layout of the matrix cores: register i of a quad's lanes = the sum of row i.
+    // The epilogue stores from lanes 0..3 of the wavefront: lane 4*b + j wants, in register i
+    // of set q, the sum that lane 4*b + i holds for batch row 4*q + j.
     __device__ __forceinline__ void fold() {
-        if (QUARTER) {
-            const uint32_t d = __float_as_uint(dot);
-            acc[0] = f32x4_t{__uint_as_float(quad_bcast<0>(d)), __uint_as_float(quad_bcast<1>(d)),
-                             __uint_as_float(quad_bcast<2>(d)), __uint_as_float(quad_bcast<3>(d))};
+        const int mine = threadIdx.x & 3;
+#pragma unroll
+        for (int q = 0; q < NSET; ++q) {
+            uint32_t r[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (4 * q + j < BS) {
+                    const uint32_t d = __float_as_uint(dot[4 * q + j]);
+                    const uint32_t t[4] = {quad_bcast<0>(d), quad_bcast<1>(d), quad_bcast<2>(d), quad_bcast<3>(d)};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) r[i] = mine == j ? t[i] : r[i];
+                }
+            }
+            acc[q] = f32x4_t{__uint_as_float(r[0]), __uint_as_float(r[1]), __uint_as_float(r[2]), __uint_as_float(r[3])};
         }
     }
 };
@@ -402,11 +406,13 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     const int K = s.Ks * s.split_k;
     const bool variant = Codec::variant(header);
 
-    MfmaPolicy<BS> pol;
-    constexpr int NSET = MfmaPolicy<BS>::NSET;
+    DotPolicy<BS> pol;
+    constexpr int NSET = DotPolicy<BS>::NSET;
 #pragma unroll
     for (int q = 0; q < NSET; ++q) pol.acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    pol.dot = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pol.dot[j] = 0.f;
+    pol.xrow = K / 2;
 
     if (active) {
         for (int kc = p; kc < per_group; kc += P) {
@@ -414,12 +420,6 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
             typename Codec::Cursor cur;
             cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
             pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
-#pragma unroll
-            for (int q = 0; q < NSET; ++q) {
-                const int batch = (lane & 3) + 4 * q;
-                pol.x0[q] = (const uint4*)(X + (size_t)(batch < BS ? batch : 0) * K + (size_t)id.k * s.Ks
-                                           + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols);
-            }
             pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
             if (variant) run_task<true>(cur, lut, pol, id.t1 - id.t0, stage_table);
