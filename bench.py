@@ -258,7 +258,7 @@ def main():
         # 28 such blocks make one Qwen2.5-7B token (attention, norms, embedding and lm_head not included)
         "bs1_tokens_per_s_28_blocks": round(1.0 / sec / 28, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
-        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{dict(huffman='HuffCodec', ans='AnsCodec', nibble='NibbleCodec')[args.algo]}, {bs}, 4> "
+        "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{dict(huffman='HuffCodec', ans='AnsCodec', nibble='NibbleCodec')[args.algo]}, {bs}, 4, {2 if args.no_group else 4}> "
                                f"{dom_name}",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),

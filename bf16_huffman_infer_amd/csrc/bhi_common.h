@@ -86,7 +86,7 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
     return s;
 }
 
-// A task is processed in segments of kSegSteps steps; the global loads of a segment (all
+// A task is processed in segments of S steps; the global loads of a segment (all
 // unconditional) are issued back to back, one whole segment before they are used.  VMEM
 // loads complete in issue order, so a load issued on demand inside a segment would make
 // its wait drain the whole queue.  Two steps per segment: on short tasks (7 steps) that is 6-12 %
@@ -97,30 +97,28 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
 // that the three rows of a window are always at +0, +256 and +512 bytes of one address.
 // Lanes sit at different rows, yet row r of lane l is always in bank l % 32: window reads
 // are conflict free.  A task stages kPrimeRows rows before its first step; every segment
-// then prefetches the next kSegRows rows if every lane has made room for them, and the
+// then prefetches the next S rows if every lane has made room for them, and the
 // following segment commits them to the ring.  A lane whose window is not staged (a
 // cheap per-step test) reads it from global memory instead.
-#ifndef BHI_SEG_STEPS
-#define BHI_SEG_STEPS 2
-#define BHI_SEG_ROWS 2
-#endif
-constexpr int kSegSteps = BHI_SEG_STEPS;
+// The segment length S is a template parameter of the walk: kSegShort or kSegLong steps,
+// with as many rows prefetched per segment.
+constexpr int kSegShort = 2;
+constexpr int kSegLong = 4;
 #ifndef BHI_RING_ROWS
 #define BHI_RING_ROWS 16
 #endif
 constexpr int kRingRows = BHI_RING_ROWS;
 constexpr int kRingRowsLog2 = kRingRows == 8 ? 3 : kRingRows == 16 ? 4 : kRingRows == 32 ? 5 : -1;
 static_assert(kRingRowsLog2 > 0, "ring of 8, 16 or 32 rows");
-constexpr int kSegRows = BHI_SEG_ROWS;          // rows prefetched per segment
 #ifndef BHI_PRIME_ROWS
 #define BHI_PRIME_ROWS 8
 #endif
 constexpr int kPrimeRows = BHI_PRIME_ROWS;      // rows staged before the first step
 constexpr int kRingSlots = kRingRows + 2;   // slots 0 and 1 are mirrored behind the last one
 constexpr int kRingWords = kRingSlots * kLanes;
-static_assert(kRingRows % kSegRows == 0 && (kRingRows & (kRingRows - 1)) == 0 && kSegRows >= 2,
+static_assert(kRingRows % kSegLong == 0 && kSegLong % kSegShort == 0 && (kRingRows & (kRingRows - 1)) == 0 && kSegShort >= 2,
               "rows are committed in aligned groups; the group at slot 0 carries both mirrored rows");
-static_assert(kPrimeRows % kSegRows == 0 && kPrimeRows >= 4 && kPrimeRows <= kRingRows, "priming stages whole groups");
+static_assert(kPrimeRows % kSegLong == 0 && kPrimeRows >= 4 && kPrimeRows <= kRingRows, "priming stages whole groups");
 
 // The rem plane is read once, front to back, 512 aligned bytes per wavefront and step:
 // loaded with the non-temporal hint its lines leave the caches first and stop displacing
@@ -189,35 +187,38 @@ struct RowRing {
         lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi - 2) << 5;
     }
 
-    // Can the next kSegRows rows be staged now?  Row r may replace row r - kRingRows once
+    // Can the next R rows be staged now?  Row r may replace row r - kRingRows once
     // no window needs it, i.e. once every lane is past it: one compare and a ballot.  Rows
-    // are staged in whole groups: rhi stays a multiple of kSegRows and a group never wraps
+    // are staged in whole groups: rhi stays a multiple of R and a group never wraps
     // around the ring.  Decided before the loads are issued so that they need not be
     // issued in vain (and so that the compiler cannot sink them behind the decision).
+    template <int R>
     __device__ __forceinline__ bool room() const {
-        const uint32_t top = rhi + kSegRows;
+        const uint32_t top = rhi + R;
         const uint32_t oldest = top > (uint32_t)kRingRows ? (top - kRingRows) << 5 : 0u;
         return rhi < nrows && ballot(pos < oldest) == 0;
     }
 
-    // The next kSegRows rows after the staged ones: one address, immediate offsets.  Rows
+    // The next R rows after the staged ones: one address, immediate offsets.  Rows
     // past the end of the block belong to the next block or to the zero pad that ends the
     // stream; they are loaded, staged, never decoded.
-    __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) const {
+    template <int R>
+    __device__ __forceinline__ void prefetch(uint32_t (&v)[R]) const {
         const uint32_t* p = bp + (size_t)rhi * kLanes;
 #pragma unroll
-        for (int j = 0; j < kSegRows; ++j) v[j] = p[j * kLanes];
+        for (int j = 0; j < R; ++j) v[j] = p[j * kLanes];
     }
 
-    __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
+    template <int R>
+    __device__ __forceinline__ void commit(const uint32_t (&v)[R]) {
         lds_u32* dst = ring + (rhi & (kRingRows - 1)) * kLanes;
 #pragma unroll
-        for (int j = 0; j < kSegRows; ++j) dst[j * kLanes] = v[j];
+        for (int j = 0; j < R; ++j) dst[j * kLanes] = v[j];
         if ((rhi & (kRingRows - 1)) == 0) {
             ring[kRingRows * kLanes] = v[0];
             ring[(kRingRows + 1) * kLanes] = v[1];
         }
-        rhi += kSegRows;
+        rhi += R;
         set_lim();
     }
 
@@ -378,7 +379,7 @@ struct NibbleCursor {
     uint32_t eptr;           // wave-uniform: escape entries consumed so far
     uint32_t next;           // wave-uniform: first step not prefetched yet
     uint32_t base4;          // wave-uniform: the base exponent in every byte
-    uint32_t cur[kSegSteps]; // the words of the segment being decoded
+    uint32_t cur[kSegLong];  // the words of the segment being decoded (one row per step)
 
     __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t*) {
         bp = words + span.base + lane;
@@ -389,19 +390,22 @@ struct NibbleCursor {
     __device__ __forceinline__ void prime_issue(uint32_t (&)[kPrimeRows]) const {}
     __device__ __forceinline__ void prime_commit(const uint32_t (&)[kPrimeRows]) const {}
     __device__ __forceinline__ void start(const uint32_t* lut) { base4 = uniform(lut[0] & 0xFFu) * 0x01010101u; }
+    template <int R>
     __device__ __forceinline__ bool room() const { return true; }
-    static_assert(kSegRows == kSegSteps, "one row per step");
 
     // rows past the last step belong to the escape list, the next block or the zero pad
-    __device__ __forceinline__ void prefetch(uint32_t (&v)[kSegRows]) {
+    template <int R>
+    __device__ __forceinline__ void prefetch(uint32_t (&v)[R]) {
         const uint32_t* p = bp + (size_t)next * kLanes;
 #pragma unroll
-        for (int j = 0; j < kSegRows; ++j) v[j] = p[j * kLanes];
-        next += kSegRows;                          // segments are prefetched in order, possibly one ahead
+        for (int j = 0; j < R; ++j) v[j] = p[j * kLanes];
+        next += R;                          // segments are prefetched in order, possibly one ahead
     }
-    __device__ __forceinline__ void commit(const uint32_t (&v)[kSegRows]) {
+    template <int R>
+    __device__ __forceinline__ void commit(const uint32_t (&v)[R]) {
+        static_assert(R <= kSegLong, "cur holds one segment");
 #pragma unroll
-        for (int j = 0; j < kSegRows; ++j) cur[j] = v[j];
+        for (int j = 0; j < R; ++j) cur[j] = v[j];
     }
 
     // pair entries in the Huffman table's format (a<<7 | b<<23) for step i of the segment

@@ -24,15 +24,15 @@ struct Shape {
     uint32_t total_words;
 };
 
-// One segment of a task: kSegSteps steps whose operands a policy has loaded into `slot`.
+// One segment of a task: S steps whose operands a policy has loaded into `slot`.
 // `Slot` holds what is loaded per step; `take(...)` hands out what the policy pipelines
 // on its own inside the compute phase; `use(...)` receives the lane's four rebuilt BF16
 // pairs (columns 0..7 of its row in step t).
-template <bool FULL, bool HAS_ESC, class Cursor, class Policy>
+template <bool FULL, bool HAS_ESC, int S, class Cursor, class Policy>
 __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut, Policy& pol,
-                                               const typename Policy::Slot (&slot)[kSegSteps], int t0, int ns) {
+                                               const typename Policy::Slot (&slot)[S], int t0, int ns) {
 #pragma unroll
-    for (int i = 0; i < kSegSteps; ++i) {
+    for (int i = 0; i < S; ++i) {
         if (FULL || t0 + i < ns) {
             const typename Policy::Piped piped = pol.take(slot[i], i, t0 + i);
             uint32_t e[4];
@@ -53,12 +53,12 @@ __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut,
 // `next`, decode `now`.  Every global load is thus issued a whole segment before its
 // first use and is unconditional apart from the row prefetch, so the compiler can count
 // the outstanding ones and make each step wait for exactly its own operands.
-template <bool HAS_ESC, class Cursor, class Policy>
+template <bool HAS_ESC, int S, class Cursor, class Policy>
 __device__ __forceinline__ void run_segment(Cursor& cur, const uint32_t* lut, Policy& pol, bool& pending,
-                                            uint32_t (&rows)[kSegRows], const typename Policy::Slot (&now)[kSegSteps],
-                                            typename Policy::Slot (&next)[kSegSteps], int seg, int next_seg, int ns) {
+                                            uint32_t (&rows)[S], const typename Policy::Slot (&now)[S],
+                                            typename Policy::Slot (&next)[S], int seg, int next_seg, int ns) {
     if (pending) cur.commit(rows);
-    pending = cur.room();
+    pending = cur.template room<S>();
     if (pending) cur.prefetch(rows);
     pol.load_full(next, next_seg);
     decode_segment<true, HAS_ESC>(cur, lut, pol, now, seg, ns);
@@ -70,17 +70,17 @@ __device__ __forceinline__ void run_segment(Cursor& cur, const uint32_t* lut, Po
 // together.  Whole segments alternate between two operand sets (one being decoded, one in
 // flight); the last whole segment reloads itself instead of running past the task.  A
 // last, shorter segment clamps its step indices and guards its steps.
-template <bool HAS_ESC, class Cursor, class Policy, class Between>
+template <bool HAS_ESC, int S, class Cursor, class Policy, class Between>
 __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between) {
-    typename Policy::Slot a[kSegSteps], b[kSegSteps];
-    const int full_end = ns - ns % kSegSteps;
-    const int last_full = full_end - kSegSteps;
+    typename Policy::Slot a[S], b[S];
+    const int full_end = ns - ns % S;
+    const int last_full = full_end - S;
     pol.prime();
     if (full_end > 0) {
         pol.load_full(a, 0);
     } else {
 #pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) pol.load(a[i], i);
+        for (int i = 0; i < S; ++i) pol.load(a[i], i);
     }
     {
         uint32_t first[kPrimeRows];
@@ -89,28 +89,28 @@ __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Polic
         cur.prime_commit(first);
     }
     cur.start(lut);
-    uint32_t rows[kSegRows];
-    bool pending = cur.room();
+    uint32_t rows[S];
+    bool pending = cur.template room<S>();
     if (pending) cur.prefetch(rows);
     int seg = 0;
     if (full_end > 0) {
         for (;;) {
-            int nx = seg + kSegSteps;
-            run_segment<HAS_ESC>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, ns);
+            int nx = seg + S;
+            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
-            nx = seg + kSegSteps;
-            run_segment<HAS_ESC>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, ns);
+            nx = seg + S;
+            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
         }
         if (seg < ns) {
 #pragma unroll
-            for (int i = 0; i < kSegSteps; ++i) pol.load(a[i], seg + i);
+            for (int i = 0; i < S; ++i) pol.load(a[i], seg + i);
         }
     }
     if (pending) cur.commit(rows);
-    if (seg < ns) decode_segment<false, HAS_ESC>(cur, lut, pol, a, seg, ns);
+    if (seg < ns) decode_segment<false, HAS_ESC, S>(cur, lut, pol, a, seg, ns);
 }
 
 // The format header (code_lengths buffer): [0] version, [1] table bits, [2] ESC code
@@ -132,10 +132,11 @@ struct StorePolicy {
         t = t < last ? t : last;
         s.rem = stream_load(rem0 + (size_t)t * kLanes);
     }
-    __device__ __forceinline__ void load_full(Slot (&s)[kSegSteps], int t0) const {
+    template <int S>
+    __device__ __forceinline__ void load_full(Slot (&s)[S], int t0) const {
         const uint2* p = rem0 + (size_t)t0 * kLanes;
 #pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) s[i].rem = stream_load(p + i * kLanes);
+        for (int i = 0; i < S; ++i) s[i].rem = stream_load(p + i * kLanes);
     }
     __device__ __forceinline__ Piped take(const Slot&, int, int) const { return Piped{}; }
     __device__ __forceinline__ void use(const Piped&, int t, const uint32_t (&w)[4]) const {
@@ -219,11 +220,12 @@ struct DotPolicy {
         s.rem = stream_load(rem0 + (size_t)t * kLanes);
         if (!PIPED) xpairs<0>(s.x, xq0 + (size_t)t * (kStepCols / 2));
     }
-    __device__ __forceinline__ void load_full(Slot (&s)[kSegSteps], int t0) const {
+    template <int S>
+    __device__ __forceinline__ void load_full(Slot (&s)[S], int t0) const {
         const uint2* pr = rem0 + (size_t)t0 * kLanes;
         const uint32_t* pq = xq0 + (size_t)t0 * (kStepCols / 2);
 #pragma unroll
-        for (int i = 0; i < kSegSteps; ++i) {
+        for (int i = 0; i < S; ++i) {
             s[i].rem = stream_load(pr + i * kLanes);
             if (!PIPED) xpairs<0>(s[i].x, pq + i * (kStepCols / 2));
         }
@@ -285,7 +287,7 @@ __device__ __forceinline__ TaskId task_of(const Shape& s, int kc) {
 }
 
 // ------------------------------------------------------------------ decode to BF16
-template <class Codec, int NW>
+template <class Codec, int NW, int S>
 __global__ __launch_bounds__(NW * kLanes)
 void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict__ A_exp,
                            uint16_t* __restrict__ Y, const uint32_t* __restrict__ offsets,
@@ -319,8 +321,8 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
     pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
     pol.yp = Y + (size_t)(kGroupRows * g + (lane & 3)) * K + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols + (lane >> 2) * kLaneCols;
     pol.last = id.t1 - id.t0 - 1;
-    if (Codec::variant(header)) run_task<true>(cur, lut, pol, id.t1 - id.t0, stage_table);
-    else run_task<false>(cur, lut, pol, id.t1 - id.t0, stage_table);
+    if (Codec::variant(header)) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_table);
+    else run_task<false, S>(cur, lut, pol, id.t1 - id.t0, stage_table);
 }
 
 // ------------------------------------------------------------------ fused decode + GEMV
@@ -361,7 +363,7 @@ __device__ __forceinline__ uint16_t finish_output(float sum, const uint16_t* __r
     return y;
 }
 
-template <class Codec, int BS, int NW>
+template <class Codec, int BS, int NW, int S>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
 void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     // The partial sums reuse the rings once every task of the block is done.
@@ -422,8 +424,8 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
             pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
             pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
-            if (variant) run_task<true>(cur, lut, pol, id.t1 - id.t0, stage_table);
-            else run_task<false>(cur, lut, pol, id.t1 - id.t0, stage_table);
+            if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_table);
+            else run_task<false, S>(cur, lut, pol, id.t1 - id.t0, stage_table);
         }
         pol.fold();
         // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
@@ -506,11 +508,19 @@ static inline int gemv_blocks(const bhi::Shape& s) {
     return (s.M / kGroupRows + gpb - 1) / gpb;
 }
 
+// Segment length of a launch.  Short segments start sooner and lose less on tasks of a
+// handful of steps: 5-10 % faster whenever every wavefront of the launch is resident at
+// once.  A launch with more wavefronts than the GPU holds (a group of weights) runs at
+// full contention for most of its time, where the smaller per-step overhead of long
+// segments wins by about 5 %.
 template <class Codec, int BS>
 static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks, hipStream_t stream) {
     using namespace bhi;
-    hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock>), dim3((unsigned)blocks), dim3(kWavesPerBlock * kLanes),
-                       0, stream, (const uint16_t*)X, grp);
+    const dim3 grid((unsigned)blocks), block(kWavesPerBlock * kLanes);
+    if ((long long)blocks * kWavesPerBlock > kTargetTasks)
+        hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegLong>), grid, block, 0, stream, (const uint16_t*)X, grp);
+    else
+        hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegShort>), grid, block, 0, stream, (const uint16_t*)X, grp);
 }
 
 template <class Codec>
@@ -579,7 +589,7 @@ static inline void launch_decode(const void* A_rem, const void* A_exp, void* Y, 
     constexpr int NW = 4;
     const long long ntasks = (long long)(s.M / kGroupRows) * s.split_k * s.nc;
     const unsigned grid = (unsigned)((ntasks + NW - 1) / NW);
-    hipLaunchKernelGGL((decode_kernel<Codec, NW>), dim3(grid), dim3(NW * kLanes), 0, st,
+    hipLaunchKernelGGL((decode_kernel<Codec, NW, kSegLong>), dim3(grid), dim3(NW * kLanes), 0, st,
                        (const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
                        (const uint32_t*)table, (const uint8_t*)header, s);
 }
