@@ -508,16 +508,18 @@ static inline int gemv_blocks(const bhi::Shape& s) {
     return (s.M / kGroupRows + gpb - 1) / gpb;
 }
 
-// Segment length of a launch.  Short segments start sooner and lose less on tasks of a
-// handful of steps: 5-10 % faster whenever every wavefront of the launch is resident at
-// once.  A launch with more wavefronts than the GPU holds (a group of weights) runs at
-// full contention for most of its time, where the smaller per-step overhead of long
-// segments wins by about 5 %.
+// Segment length of a launch.  Short segments start sooner and lose less on short tasks:
+// 5-10 % faster whenever every wavefront of the launch is resident at once, and on tasks
+// of 8 or 16 steps in any case.  A launch with more wavefronts than the GPU holds (a group
+// of weights) runs at full contention for most of its time; there, on long tasks (28
+// steps), the smaller per-step overhead of long segments wins by about 5 %.
+constexpr int kLongTaskSteps = 24;
 template <class Codec, int BS>
 static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks, hipStream_t stream) {
     using namespace bhi;
     const dim3 grid((unsigned)blocks), block(kWavesPerBlock * kLanes);
-    if ((long long)blocks * kWavesPerBlock > kTargetTasks)
+    const Shape& s0 = grp.m[0].s;
+    if ((long long)blocks * kWavesPerBlock > kTargetTasks && s0.steps / s0.nc >= kLongTaskSteps)
         hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegLong>), grid, block, 0, stream, (const uint16_t*)X, grp);
     else
         hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegShort>), grid, block, 0, stream, (const uint16_t*)X, grp);
