@@ -170,12 +170,13 @@ __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
 //
 // acc += x[q].lo * w.lo + x[q].hi * w.hi, where x[q] is the X pair held by lane q of this
 // lane's quad: v_dot2c_f32_bf16 with the quad broadcast folded into its DPP operand (the
-// compiler keeps a separate v_mov_dpp when given the builtins).  `x` must come straight
-// from a load: a VALU write to it right before a DPP read would need two wait states.
+// compiler keeps a separate v_mov_dpp when given the builtins).  A VALU write to `x` right
+// before a DPP read of it needs two wait states, and the compiler cannot see the DPP read
+// inside the asm: the first of the four products of an X pair (Q = 0) carries them.
 template <int Q>
 __device__ __forceinline__ void dot_quad(float& acc, uint32_t x, uint32_t w) {
     static_assert(Q >= 0 && Q < 4, "a quad has four lanes");
-    if (Q == 0) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
+    if (Q == 0) asm("s_nop 1\n\tv_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
     if (Q == 1) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
     if (Q == 2) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
     if (Q == 3) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
