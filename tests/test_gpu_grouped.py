@@ -43,6 +43,28 @@ def test_grouped_equals_single_launches(cuda, algo, bs, K, Ms):
         torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
 
 
+@pytest.mark.parametrize("algo", ["huffman", "ans", "nibble"])
+@pytest.mark.parametrize("bs", [1, 5])
+def test_oversubscribed_group_of_long_tasks(cuda, algo, bs):
+    """Two 12800x3072 weights are 2 x 3200 tasks of 24 steps: more wavefronts than the GPU
+    holds at once, which is the case the library serves with its long-segment kernels; a
+    weight alone runs the short-segment ones.  Same arithmetic, same order: equal bits."""
+    from bf16_huffman_infer_amd import _lib
+    from bf16_huffman_infer_amd.functional import linear_grouped
+    M, K = 12800, 3072
+    assert _lib.load().bhi_chunks_per_group(M, K, 1) == 1 and 2 * (M // 4) > 6144 and K // 128 >= 24
+    g = torch.Generator(device="cuda").manual_seed(11)
+    ws = [(torch.randn(M, K, generator=g, device="cuda") * 0.02).bfloat16() for _ in range(2)]
+    mods = [_cls(algo).compress(w).cuda() for w in ws]
+    x = torch.randn(bs, K, generator=g, device="cuda").bfloat16()
+    got = linear_grouped(x, mods, [None, None])
+    for w, mod, y in zip(ws, mods, got):
+        single = torch.nn.functional.linear(x, mod)
+        assert torch.equal(y.view(torch.int16), single.view(torch.int16))
+        ref = x.float() @ w.float().T
+        torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+
+
 def test_grouped_split_k_and_leading_dims(cuda):
     from bf16_huffman_infer_amd.functional import HuffmanWeight, linear_grouped
     K = 12288                                          # split_k = 3
