@@ -17,7 +17,6 @@ reported as the length of the common prefix rather than asserted).
 """
 import argparse
 import json
-import math
 import os
 import sys
 import time
