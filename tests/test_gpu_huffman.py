@@ -125,6 +125,24 @@ def test_full_size_layers_round_trip(cuda, algo, kind, M, K):
         torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
 
 
+@pytest.mark.parametrize("algo", ["huffman", "nibble"])
+def test_vocabulary_sized_weight(cuda, algo):
+    """151936 rows (the lm_head of the decoder configuration): 37 984 row groups, the largest
+    M of any configuration; row and byte indices go past 2**27 and 2**29."""
+    from bf16_huffman_infer_amd.functional import HuffmanWeight, NibbleWeight
+    M, K = 151936, 4096
+    g = torch.Generator(device="cuda").manual_seed(5)
+    w = (torch.randn(M, K, generator=g, device="cuda") * 0.02).bfloat16()
+    mod = (HuffmanWeight if algo == "huffman" else NibbleWeight).compress(w).cuda()
+    got = mod.get_weight()
+    assert torch.equal(got.view(torch.int16), w.view(torch.int16))
+    del got
+    x = torch.randn(2, K, generator=g, device="cuda").bfloat16()
+    y = torch.nn.functional.linear(x, mod)
+    ref = x.float() @ w.float().T
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+
+
 @pytest.mark.parametrize("algo", ["huffman", "ans"])
 def test_long_incompressible_tasks_outrun_the_row_ring(cuda, algo):
     """128-step tasks whose exponents are uniform over 39 values: every pair costs about

@@ -72,3 +72,14 @@ def test_package_does_not_import_the_oracle():
             "assert not [m for m in sys.modules if m == 'oracle' or m.startswith('oracle.')]")
     subprocess.run([sys.executable, "-c", code], check=True, cwd=__import__("os").path.dirname(
         __import__("os").path.dirname(__import__("os").path.abspath(__file__))))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build measures one GPU; asking the benchmark for more must say so and stop."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stderr + r.stdout)
