@@ -32,7 +32,9 @@ STD = 0.02
 # runs of this script, each scaled by the same counter's reading for the 256 MiB calibration
 # copy below.  Keyed by (algo, batch, launch): "single" = one 18944x3584 matrix, "group" =
 # gate_proj + up_proj in one launch; None where it has not been measured.
-MEASURED_TRAFFIC = {("huffman", 1, "single"): 94_620_000, ("huffman", 1, "group"): 199_860_000}
+MEASURED_TRAFFIC = {("huffman", 1, "single"): 94_620_000, ("huffman", 1, "group"): 199_860_000,
+                    ("nibble", 1, "single"): 104_700_000, ("nibble", 1, "group"): 223_520_000,
+                    ("ans", 1, "single"): 96_270_000, ("ans", 1, "group"): 205_720_000}
 
 
 def make_weight(M, K, seed, device):
