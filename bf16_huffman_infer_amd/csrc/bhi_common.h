@@ -355,7 +355,8 @@ struct AnsCursor : RowRing {
     __device__ __forceinline__ uint32_t pair(const uint32_t* __restrict__ table) {
         const uint32_t a = symbol(table);
         const uint32_t b = symbol(table);
-        return ((a >> 17) & 0x7F80u) | ((b >> 1) & 0x7F800000u);
+        // the two symbols (byte 3 of the table words) to bytes 0 and 2, then to bits 7 and 23
+        return __builtin_amdgcn_perm(b, a, 0x0C070C03u) << 7;
     }
 
     template <bool UNUSED>
