@@ -17,8 +17,8 @@
 Pins.  Huffman: the cascade decodes every code back to its symbol (checked by
 ``decode_code`` over all symbols), codes are prefix-free with Kraft sum 1, lengths are
 within 1 bit of entropy on unperturbed inputs.  The exact tie-breaking of the
-reference's heap is NOT reproduced (it does not affect decoded weights): "parity
-unpinned" for byte-identical tables.  rANS: the worked example of ``ans.py:152``
+reference's heap is NOT reproduced (it does not affect decoded weights):
+"parity unpinned" for byte-identical tables.  rANS: the worked example of ``ans.py:152``
 (counts x16 exactly -> freq {1:96, 2:32, 3:32, 6..13:16}), sum/positivity/prefix
 invariants, slot bijection.
 """
