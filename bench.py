@@ -104,6 +104,37 @@ def time_launches(fn, n, warmup, launches_per_graph=1):
     return start.elapsed_time(stop) * 1e-3 / (replays * launches_per_graph)
 
 
+def load_only(launch_bytes, args, device):
+    """The ceiling measured in the same run: a kernel that only loads the bytes of one
+    18944x3584 launch (as many wavefronts as that layer has tasks, four 16-byte loads in
+    flight per lane, nothing kept), rotating over >= 640 MB like the per-layer timings."""
+    from bf16_huffman_infer_amd import _lib
+    lib = _lib.load()
+    waves = 18944 // 4                                   # one wavefront per task of the layer
+    n = max(2, -(-ROTATE_BYTES // launch_bytes))
+    stride = -(-launch_bytes // 256) * 256
+    buf = torch.empty(n * stride, dtype=torch.uint8, device=device).random_(0, 255)
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+    res = {"wavefronts": waves, "unit": "GB/s"}
+    for name, nt in (("non_temporal", 1), ("plain", 0)):
+        st = {"i": 0, "bytes": 0}
+
+        def one(st=st, nt=nt):
+            i = st["i"] % n
+            st["i"] += 1
+            got = lib.bhi_stream_read(buf.data_ptr() + i * stride, launch_bytes, waves, nt, sink.data_ptr(),
+                                      torch.cuda.current_stream().cuda_stream)
+            if got <= 0:
+                raise RuntimeError(f"bhi_stream_read failed: {got}")
+            st["bytes"] = got
+        t = time_launches(one, max(100, args.steps), args.warmup, launches_per_graph=n)
+        res[name] = round(st["bytes"] / t / 1e9, 1)
+        res["bytes_per_launch"] = st["bytes"]
+        res[f"us_per_launch_{name}"] = round(t * 1e6, 2)
+    res["frac_of_peak"] = round(res["non_temporal"] / HBM_PEAK_GBS, 4)
+    return res
+
+
 def cpu_baseline(rows=18944, K=3584, reps=5):
     """Reference layout + reference decoder (numpy) + host matmul on a slice of gate_proj."""
     import numpy as np
@@ -272,6 +303,7 @@ def main():
                           "traffic": MEASURED_TRAFFIC.get((args.algo, bs, "single")),
                           "bytes_per_launch": single_bytes, "us_per_launch": round(t_single * 1e6, 2)},
     }
+    out["load_only"] = load_only(single_bytes, args, device)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -25,6 +25,7 @@ _SIGNATURES = {
     "bhi_constants": (_i32, [ctypes.POINTER(ctypes.c_int32), _i32]),
     "bhi_chunks_per_group": (_i32, [_i32, _i32, _i32]),
     "bhi_last_error_string": (ctypes.c_char_p, []),
+    "bhi_stream_read": (_i64, [_vp, _i64, _i32, _i32, _vp, _vp]),
     "bhi_gemv_bf16_huffman": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,
                                      _i32, _i32, _i32, _i32, _vp]),
     "bhi_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,

@@ -34,3 +34,51 @@ extern "C" int bhi_chunks_per_group(int M, int Ks, int split_k) {
     if (M < bhi::kGroupRows || Ks < bhi::kStepCols || split_k < 1) return bhi_fail(BHI_EINVAL, "bad shape");
     return bhi::chunks_per_group(M, Ks, split_k);
 }
+
+// A loop that only loads: `wavefronts` wavefronts each stream a contiguous span of `src`
+// with four 16-byte loads in flight per lane and keep nothing.  It measures what this GPU
+// delivers to a kernel with the fused GEMV's shape (one wavefront per task, a few KB in
+// flight each) when there is no decode work at all: the ceiling the GEMV sits under.
+namespace bhi {
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+template <bool NT>
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint32_t* __restrict__ src, long long words_per_wave,
+                                                           uint32_t* __restrict__ sink) {
+    const int lane = threadIdx.x & (kLanes - 1);
+    const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const uint32_t* base = src + wave * words_per_wave;
+    uint32_t acc = 0;
+    long long o = 0;
+    for (; o + 4 * 4 * kLanes <= words_per_wave; o += 4 * 4 * kLanes) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const u32x4_t* q = (const u32x4_t*)(base + o + u * 4 * kLanes) + lane;
+            const u32x4_t v = NT ? __builtin_nontemporal_load(q) : *q;
+            acc += v.x ^ v.y ^ v.z ^ v.w;
+        }
+    }
+    for (; o + 4 * kLanes <= words_per_wave; o += 4 * kLanes) {      // the last, shorter iteration
+        const u32x4_t* q = (const u32x4_t*)(base + o) + lane;
+        const u32x4_t v = NT ? __builtin_nontemporal_load(q) : *q;
+        acc += v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9E3779B9u) sink[0] = acc;     // keeps the loads alive; not taken on real data
+}
+}  // namespace bhi
+
+extern "C" int64_t bhi_stream_read(const void* src, int64_t bytes, int wavefronts, int nontemporal, void* sink, void* stream) {
+    if (!src || !sink) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (wavefronts < 4 || wavefronts % 4 != 0 || bytes < 0) return bhi_fail(BHI_EINVAL, "wavefronts must be a positive multiple of 4");
+    const long long chunk = 4 * bhi::kLanes;                           // words of one load of a wavefront
+    const long long words_per_wave = bytes / 4 / wavefronts / chunk * chunk;
+    if (words_per_wave > 0) {
+        if (nontemporal)
+            hipLaunchKernelGGL(bhi::stream_read_kernel<true>, dim3((unsigned)(wavefronts / 4)), dim3(256), 0, (hipStream_t)stream,
+                               (const uint32_t*)src, words_per_wave, (uint32_t*)sink);
+        else
+            hipLaunchKernelGGL(bhi::stream_read_kernel<false>, dim3((unsigned)(wavefronts / 4)), dim3(256), 0, (hipStream_t)stream,
+                               (const uint32_t*)src, words_per_wave, (uint32_t*)sink);
+        if (int rc = bhi_launch_status("stream_read")) return -(int64_t)(rc > 0 ? rc : -rc);
+    }
+    return words_per_wave * 4 * wavefronts;
+}

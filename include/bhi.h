@@ -173,6 +173,15 @@ int bhi_reference_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_w
                              void* Y, const void* offsets, const void* LUT,
                              int split_k, int M, int Ks, void* stream);
 
+/* No counterpart in the reference: a measurement helper.  Enqueues a kernel in which
+ * `wavefronts` wavefronts (a positive multiple of 4) each load a contiguous span of `src`
+ * (four 16-byte loads in flight per lane, with or without the non-temporal hint) and keep
+ * nothing: the rate at which this GPU feeds a kernel of the fused GEMV's shape when there is
+ * nothing to decode.  `src` must be 16-byte aligned; `sink` is 4 bytes of device memory that
+ * are not written in practice.  Returns the number of bytes the launch reads (`bytes` rounded
+ * down to whole 1 KB loads of every wavefront), or a negative error. */
+int64_t bhi_stream_read(const void* src, int64_t bytes, int wavefronts, int nontemporal, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

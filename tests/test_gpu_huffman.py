@@ -212,3 +212,20 @@ def test_linear_with_no_rows(cuda):
     assert y.shape == (0, 128) and y.dtype == torch.bfloat16
     y = torch.nn.functional.linear(torch.empty(2, 0, 1024, dtype=torch.bfloat16, device="cuda"), mod)
     assert y.shape == (2, 0, 128)
+
+
+def test_stream_read_helper(cuda):
+    """The load-only measurement kernel: reads whole 1 KB loads per wavefront, rejects bad arguments."""
+    from bf16_huffman_infer_amd import _lib
+    lib = _lib.load()
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    for nt in (0, 1):
+        assert lib.bhi_stream_read(buf.data_ptr(), buf.numel(), 64, nt, sink.data_ptr(), st) == 1 << 20
+        assert lib.bhi_stream_read(buf.data_ptr(), (1 << 20) - 1, 64, nt, sink.data_ptr(), st) == (1 << 20) - 64 * 1024
+    assert lib.bhi_stream_read(buf.data_ptr(), 100, 64, 1, sink.data_ptr(), st) == 0          # nothing to launch
+    torch.cuda.synchronize()
+    assert sink.item() == 0
+    assert lib.bhi_stream_read(buf.data_ptr(), buf.numel(), 6, 1, sink.data_ptr(), st) < 0
+    assert lib.bhi_stream_read(None, buf.numel(), 64, 1, sink.data_ptr(), st) < 0
