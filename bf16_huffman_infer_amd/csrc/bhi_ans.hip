@@ -16,6 +16,7 @@ constexpr int kAnsInitRows = 2;                 // rows 0, 1 of a lane: its init
 
 struct AnsCodec {
     using Cursor = AnsCursor;
+    static constexpr bool kPersistent = true;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = kAnsTableWords;
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__) { return false; }
 };

@@ -14,6 +14,7 @@ constexpr uint32_t kNibbleEsc = 15;
 
 struct NibbleCodec {
     using Cursor = NibbleCursor;
+    static constexpr bool kPersistent = false;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = 4;          // base and flags, one 16-byte copy
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ lut) {
         return uniform(((const uint32_t*)lut)[1]) != 0;

@@ -168,18 +168,25 @@ __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
 //   batch 5..8  that would be 8 * bs registers: they are fetched XAHEAD steps ahead instead,
 //               right after the step that used their registers (X is cache resident).
 //
-// acc += x[q].lo * w.lo + x[q].hi * w.hi, where x[q] is the X pair held by lane q of this
-// lane's quad: v_dot2c_f32_bf16 with the quad broadcast folded into its DPP operand (the
-// compiler keeps a separate v_mov_dpp when given the builtins).  A VALU write to `x` right
-// before a DPP read of it needs two wait states, and the compiler cannot see the DPP read
-// inside the asm: the first of the four products of an X pair (Q = 0) carries them.
-template <int Q>
-__device__ __forceinline__ void dot_quad(float& acc, uint32_t x, uint32_t w) {
-    static_assert(Q >= 0 && Q < 4, "a quad has four lanes");
-    if (Q == 0) asm("s_nop 1\n\tv_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
-    if (Q == 1) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
-    if (Q == 2) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
-    if (Q == 3) asm("v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(w));
+// acc += sum over q of x[q].lo * w[q].lo + x[q].hi * w[q].hi, where x[q] is the X pair held by
+// lane q of this lane's quad: four v_dot2c_f32_bf16 with the quad broadcast folded into their
+// DPP operand (the compiler keeps a separate v_mov_dpp when given the builtins).  A VALU
+// write to `x` right before a DPP read of it needs two wait states, and the compiler cannot
+// see the DPP reads inside the asm.  All four reads of `x` therefore sit in ONE asm statement
+// behind one s_nop: nothing the compiler emits (a register copy of `x`, say) can land
+// between a write of `x` and an unprotected read.  The other side of the statement has a
+// hazard of its own: a VALU instruction that is not the same dot product must not read
+// `acc` within three wait states of the write, and the compiler, which does not see a dot
+// product here, will happily copy `acc` to another register right behind the statement
+// (wrong sums, in whichever batch row the copy happened to hit).  Hence the closing s_nop.
+__device__ __forceinline__ void dot_quad4(float& acc, uint32_t x, const uint32_t (&w)[4]) {
+    asm("s_nop 1\n\t"
+        "v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf\n\t"
+        "v_dot2c_f32_bf16_dpp %0, %1, %3 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_dot2c_f32_bf16_dpp %0, %1, %4 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_dot2c_f32_bf16_dpp %0, %1, %5 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 2"
+        : "+v"(acc) : "v"(x), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
 }
 
 template <int BS>
@@ -216,10 +223,12 @@ struct DotPolicy {
             for (int i = 0; i < XAHEAD; ++i) xload(xr[i], i);
         }
     }
-    __device__ __forceinline__ void load(Slot& s, int t) const {
-        t = t < last ? t : last;
-        s.rem = stream_load(rem0 + (size_t)t * kLanes);
-        if (!PIPED) xpairs<0>(s.x, xq0 + (size_t)t * (kStepCols / 2));
+    __device__ __forceinline__ void load(Slot& s, int t) const { load_at(s, rem0, xq0, last, t); }
+    // step t (clamped to last_) of the task whose first step sits at r0 / x0
+    __device__ __forceinline__ void load_at(Slot& s, const uint2* r0, const uint32_t* x0, int last_, int t) const {
+        t = t < last_ ? t : last_;
+        s.rem = stream_load(r0 + (size_t)t * kLanes);
+        if (!PIPED) xpairs<0>(s.x, x0 + (size_t)t * (kStepCols / 2));
     }
     template <int S>
     __device__ __forceinline__ void load_full(Slot (&s)[S], int t0) const {
@@ -245,12 +254,7 @@ struct DotPolicy {
             const uint32_t xb[4] = {xs.x, xs.y, xs.z, xs.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                if (4 * q + j < BS) {
-                    dot_quad<0>(dot[4 * q + j], xb[j], w[0]);
-                    dot_quad<1>(dot[4 * q + j], xb[j], w[1]);
-                    dot_quad<2>(dot[4 * q + j], xb[j], w[2]);
-                    dot_quad<3>(dot[4 * q + j], xb[j], w[3]);
-                }
+                if (4 * q + j < BS) dot_quad4(dot[4 * q + j], xb[j], w);
             }
         }
         if (PIPED) xload(xr[s.i % XAHEAD], s.t + XAHEAD);
@@ -486,6 +490,8 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
 
 }  // namespace bhi
 
+#include "bhi_persist.h"
+
 static inline int check_shape(int split_k, int M, int Ks, int64_t exp_words, bhi::Shape* s) {
     using namespace bhi;
     if (split_k < 1 || M < kGroupRows || M % kGroupRows != 0 || Ks < kStepCols || Ks % kStepCols != 0)
@@ -528,6 +534,9 @@ static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks,
 
 template <class Codec>
 static inline void launch_gemv_batch(int batch, const void* X, const bhi::Group& grp, int blocks, hipStream_t st) {
+    if constexpr (Codec::kPersistent) {
+        if (try_launch_persist<Codec>(batch, X, grp, st)) return;
+    }
     switch (batch) {
         case 1: launch_gemv<Codec, 1>(X, grp, blocks, st); break;
         case 2: launch_gemv<Codec, 2>(X, grp, blocks, st); break;
