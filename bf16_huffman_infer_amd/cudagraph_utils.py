@@ -13,6 +13,7 @@ needs from them.
 :class:`GraphedCallable` is the model-independent part: any function of tensors whose
 launches stay on the current stream can be recorded with it.
 """
+import inspect
 from typing import Callable, Sequence
 
 import torch
@@ -76,11 +77,29 @@ def _max_cache_len(cache) -> int:
     return int(cache.max_cache_len)
 
 
-def apply_graphed(model, cache, replace_generate: bool = True) -> None:
+def _accepted(fn: Callable, kwargs: dict) -> dict:
+    """``kwargs`` without the names ``fn`` does not take (everything when it has ``**kwargs``).
+
+    ``forward`` and ``generate`` of transformers models gained and lost keywords over the
+    releases (``cache_position``, ``disable_compile``, ``output_attentions`` ...); the adapter
+    passes what the installed release understands instead of pinning one."""
+    try:
+        params = inspect.signature(fn).parameters
+    except (TypeError, ValueError):
+        return kwargs
+    if any(p.kind is inspect.Parameter.VAR_KEYWORD for p in params.values()):
+        return kwargs
+    return {k: v for k, v in kwargs.items() if k in params}
+
+
+def apply_graphed(model, cache, replace_generate: bool = True, recorder=None) -> None:
     """Patch ``model.forward`` in place: one-token calls replay a graph, longer calls
     (prefill) run eagerly; both write into ``cache``.  With ``replace_generate`` the
     model's ``generate`` resets and passes that cache on every call
-    (reference ``cudagraph_utils.py:11-80``)."""
+    (reference ``cudagraph_utils.py:11-80``).
+
+    ``recorder(fn, sample_args)`` turns the one-token step into the callable that replays it;
+    the default is :class:`GraphedCallable`."""
     from transformers.modeling_outputs import CausalLMOutputWithPast
 
     _old_forward = model.forward
@@ -91,7 +110,7 @@ def apply_graphed(model, cache, replace_generate: bool = True) -> None:
 
     def _forward(input_ids, attention_mask, position_ids, cache_position):
         with torch.no_grad():
-            return _old_forward(
+            return _old_forward(**_accepted(_old_forward, dict(
                 input_ids=input_ids,
                 attention_mask=attention_mask,
                 position_ids=position_ids,
@@ -101,7 +120,7 @@ def apply_graphed(model, cache, replace_generate: bool = True) -> None:
                 use_cache=True,
                 cache_position=cache_position,
                 return_dict=True,
-            ).logits
+            ))).logits
 
     zero = torch.zeros((), dtype=dtype, device=device)
     minus_inf = torch.full((), float("-inf"), dtype=dtype, device=device)
@@ -116,7 +135,7 @@ def apply_graphed(model, cache, replace_generate: bool = True) -> None:
         return _forward(input_ids, mask, cache_position.view(1, 1), cache_position)
 
     # recorded at the last cache slot so that the warm-up runs do not disturb a prompt
-    step = GraphedCallable(_step, (
+    step = (recorder or GraphedCallable)(_step, (
         torch.zeros(1, 1, dtype=torch.int64, device=device),
         torch.tensor([max_len - 1], dtype=torch.int64, device=device),
     ))
@@ -141,7 +160,14 @@ def apply_graphed(model, cache, replace_generate: bool = True) -> None:
 
         def generate(*args, **kwargs):
             cache.reset()
-            return _old_generate(*args, past_key_values=cache, disable_compile=True, **kwargs)
+            # `disable_compile` exists where generate() would otherwise compile the decode
+            # step itself; releases without it do not need it
+            extra = _accepted(_old_generate, dict(disable_compile=True))
+            if extra and 'disable_compile' not in inspect.signature(_old_generate).parameters:
+                from transformers import GenerationConfig
+                if not hasattr(GenerationConfig(), 'disable_compile'):
+                    extra = {}
+            return _old_generate(*args, past_key_values=cache, **extra, **kwargs)
 
         model.generate = generate
 

@@ -44,6 +44,7 @@ __all__ = [
     "convert_all_linear",
     "convert",
     "load_compressed_state_dict",
+    "check_layout",
 ]
 
 
@@ -54,6 +55,17 @@ def _lane_order(plane: Tensor, split_k: int) -> Tensor:
     G, S = M // GROUP_ROWS, Ks // STEP_COLS
     x = plane.view(G, GROUP_ROWS, split_k, S, STEP_COLS // LANE_COLS, LANE_COLS)     # g i k t b j
     return x.permute(2, 0, 3, 4, 1, 5).reshape(split_k, G, S, LANES, LANE_COLS)
+
+
+def _promote_single_split(A_rem: Tensor, offsets: Tensor):
+    """A weight stored without the leading split dimension (``rem`` ``[M, N]``, ``offsets`` one
+    rank lower as well) is a single split: the reference's ``mv_*`` accept that older form
+    (``functional.py:33-36, 421-424``)."""
+    if A_rem.dim() == 2:
+        A_rem = A_rem[None, :, :]
+        if offsets.dim() == 1:
+            offsets = offsets[None, :]
+    return A_rem, offsets
 
 
 def _check_weight_call(A_rem: Tensor, A_exp: Tensor, X: Tensor):
@@ -73,6 +85,7 @@ def mv_huffman(
     code_lengths: Tensor,
 ) -> Tensor:
     """Y[b, :] = W @ X[b, :] for b < 8 with W held compressed (reference ``functional.py:28-63``)."""
+    A_rem, offsets = _promote_single_split(A_rem, offsets)
     split_k, M, N = A_rem.shape
     X = X.view(-1, split_k, N)
     _check_weight_call(A_rem, A_exp, X)
@@ -85,6 +98,7 @@ def mv_huffman(
 
 def mv_ans(A_rem: Tensor, A_exp: Tensor, X: Tensor, offsets: Tensor, LUT: Tensor) -> Tensor:
     """rANS counterpart of :func:`mv_huffman` (reference ``functional.py:414-444``)."""
+    A_rem, offsets = _promote_single_split(A_rem, offsets)
     split_k, M, N = A_rem.shape
     X = X.view(-1, split_k, N)
     _check_weight_call(A_rem, A_exp, X)
@@ -319,6 +333,9 @@ class NibbleCodec:
         counts = counts.to(torch.int64).cpu()
         assert counts.numel() == 256
         cover = counts.unfold(0, self.WINDOW, 1).sum(-1)          # cover[b] = counts[b : b + 15]
+        # base + 15 (the escape nibble) must stay below 256: the decoder adds the base to four
+        # nibbles with one 32-bit add, and a carry would spill into the neighbouring exponent
+        cover = cover[:256 - self.WINDOW]
         self.base = int(torch.argmax(cover).item())               # first best window
         self.has_escapes = int(cover[self.base].item()) != int(counts.sum().item())
 
@@ -433,6 +450,12 @@ class LinearGroup:
         for m in self.members:
             m._group = self
 
+    def _biases_fit(self, input: Tensor) -> bool:
+        """The grouped launch adds BF16 biases on the input's device; anything else takes the
+        members' own path (``output += bias``), as an ungrouped module would."""
+        return all(m.bias is None or (m.bias.dtype == torch.bfloat16 and m.bias.device == input.device)
+                   for m in self.members)
+
     def dissolve(self) -> None:
         for m in self.members:
             m._group = None
@@ -442,7 +465,7 @@ class LinearGroup:
         if index == 0:
             self._input = self._outputs = None
             rows = input.numel() // input.shape[-1] if input.dim() >= 2 else MAX_FUSED_BATCH + 1
-            if self.uniform and input.is_cuda and rows <= MAX_FUSED_BATCH:
+            if self.uniform and input.is_cuda and rows <= MAX_FUSED_BATCH and self._biases_fit(input):
                 self._outputs = linear_grouped(input, [m.weight for m in self.members],
                                                [m.bias for m in self.members])
                 self._input = input
@@ -529,6 +552,39 @@ def linear_nibble(input: Tensor, weight: NibbleWeight, bias: Optional[Tensor] = 
     return _linear_compressed(input, weight, bias, fused)
 
 
+def check_layout(weight: "HuffmanWeight") -> None:
+    """Raises unless ``weight``'s buffers are in THIS package's task layout.
+
+    A weight saved by the reference package has the same buffer names, dtypes and (for rANS)
+    shapes, but its ``offsets`` are per row and its stream has no zero tail: the kernels would
+    read it as garbage, past the end of ``exp``.  Checked: the format header (Huffman), unused
+    chunk slots of ``offsets`` are 0, offsets are aligned and ascending in task order, the last
+    task ends in front of the tail pad, and the tail pad is zero."""
+    consts = _lib.constants()
+    lib = _lib.load()
+    hint = ('; a weight compressed by the reference package must be converted with '
+            'bf16_huffman_infer_amd.reference_format.transcode_reference_weight')
+    rem, exp, offsets = weight.rem, weight.exp, weight.offsets
+    if rem.dim() != 3 or offsets.dim() != 2 or tuple(offsets.shape) != tuple(rem.shape[:2]):
+        raise RuntimeError(f'compressed weight: rem {tuple(rem.shape)} / offsets {tuple(offsets.shape)} do not fit' + hint)
+    split_k, M, Ks = rem.shape
+    if isinstance(weight, HuffmanWeight) and hasattr(weight, 'LUT1'):
+        header = weight.code_lengths.flatten()[:2].tolist()
+        if weight.LUT1.numel() != 4 << consts['table_bits'] or header != [consts['format_version'], consts['table_bits']]:
+            raise RuntimeError('compressed weight: Huffman tables are not in this package\'s format' + hint)
+    if M % GROUP_ROWS or Ks % STEP_COLS:
+        raise RuntimeError(f'compressed weight: {M}x{split_k * Ks} does not fit the task layout' + hint)
+    nc = lib.bhi_chunks_per_group(M, Ks, split_k)
+    pad, align = consts['tail_pad_words'], consts['align_words']
+    off = offsets.reshape(split_k, M // GROUP_ROWS, GROUP_ROWS).to(torch.int64)
+    used = off[:, :, :nc].flatten()
+    ok = (exp.numel() >= pad and not bool(off[:, :, nc:].any()) and not bool((used % align).any())
+          and bool((used[1:] > used[:-1]).all()) and int(used[0]) == 0 and int(used[-1]) < exp.numel() - pad
+          and not bool(exp[exp.numel() - pad:].any()))
+    if not ok:
+        raise RuntimeError('compressed weight: offsets / exp are not in this package\'s task layout' + hint)
+
+
 def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool = True):
     """Load the ``state_dict()`` of a converted model into a freshly built, unconverted one.
 
@@ -551,6 +607,7 @@ def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool 
             nibble = int(state_dict[f'{name}.weight.LUT'][2]) == NibbleWeight.MAGIC
             cls = NibbleWeight if nibble else ANSWeight
         weight = cls(**{k: state_dict[f'{name}.weight.{k}'] for k in keys})
+        check_layout(weight)
         split_k, M, Ks = weight.rem.shape
         if (M, split_k * Ks) != (module.out_features, module.in_features):
             raise RuntimeError(f'{name}: compressed weight is {M}x{split_k * Ks}, '

@@ -7,7 +7,7 @@ The vectors pin the table-fill rule and the decoder cascade of the numpy restate
 against real reference tables (its heap tie-breaks and perturbation trajectory cannot be
 derived from invariants).
 """
-import importlib.util
+import types
 import json
 import os
 import sys
@@ -44,9 +44,12 @@ def histograms():
 
 
 def main():
-    spec = importlib.util.spec_from_file_location("reference_huffman", REF)
-    mod = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(mod)
+    # Run the SOURCE text: the import machinery would pick the reference's shipped bytecode
+    # cache (__pycache__/*.pyc) whenever its header matches the source file.
+    mod = types.ModuleType("reference_huffman")
+    mod.__file__ = REF
+    with open(REF) as fh:
+        exec(compile(fh.read(), REF, "exec"), mod.__dict__)
     vectors = {}
     for name, counts in histograms().items():
         enc = mod.LUTHuffmanEncoder()

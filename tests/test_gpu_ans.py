@@ -62,7 +62,7 @@ def test_fused_gemv_matches_fp32(cuda, kind, M, K, n, bs):
     y = torch.nn.functional.linear(x, mod)
     assert y.shape == (bs, M) and y.dtype == torch.bfloat16
     ref = x.float() @ w.cuda().float().T
-    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
 
 
 def test_large_batch_falls_back_to_decode_then_gemm(cuda):

@@ -67,7 +67,7 @@ def test_fused_gemv_matches_fp32(cuda, kind, M, K, n, bs):
     y = torch.nn.functional.linear(x, mod)
     assert y.shape == (bs, M) and y.dtype == torch.bfloat16
     ref = x.float() @ w.cuda().float().T
-    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
 
 
 def test_large_batch_falls_back_to_decode_then_gemm(cuda):
@@ -118,11 +118,11 @@ def test_full_size_layers_round_trip(cuda, algo, kind, M, K):
     ratio = sum(b.numel() * b.element_size() for b in mod.buffers()) / (2 * M * K)
     # short tasks (7 steps for 4608x3584) pay the 64-bit rANS state flush per lane
     assert ratio < (0.75 if algo == "huffman" else 0.78), ratio
-    for bs in (1, 8):
+    for bs in (1, 2, 4, 8):
         x = torch.randn(bs, K, generator=g, device="cuda").bfloat16()
         y = torch.nn.functional.linear(x, mod)
         ref = x.float() @ w.float().T
-        torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+        torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("algo", ["huffman", "nibble"])
@@ -140,7 +140,7 @@ def test_vocabulary_sized_weight(cuda, algo):
     x = torch.randn(2, K, generator=g, device="cuda").bfloat16()
     y = torch.nn.functional.linear(x, mod)
     ref = x.float() @ w.float().T
-    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("algo", ["huffman", "ans"])
@@ -162,7 +162,7 @@ def test_long_incompressible_tasks_outrun_the_row_ring(cuda, algo):
     x = torch.randn(3, K, generator=g).bfloat16().cuda()
     y = torch.nn.functional.linear(x, mod)
     ref = x.float() @ w.cuda().float().T
-    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()))
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("algo", ["huffman", "ans", "nibble"])
@@ -229,3 +229,17 @@ def test_stream_read_helper(cuda):
     assert sink.item() == 0
     assert lib.bhi_stream_read(buf.data_ptr(), buf.numel(), 6, 1, sink.data_ptr(), st) < 0
     assert lib.bhi_stream_read(None, buf.numel(), 64, 1, sink.data_ptr(), st) < 0
+
+
+def test_convert_keeps_the_dense_layer_when_compression_does_not_shrink_it(cuda, capsys):
+    """Weights of random bits have nothing to compress: ratio >= 1, and ``convert`` hands back the
+    original ``nn.Linear`` with the reference's warning (reference functional.py:362-365, 370-373)."""
+    from bf16_huffman_infer_amd.functional import convert
+    lin = torch.nn.Linear(512, 256, bias=False).bfloat16()
+    w = random_bits_weight(256, 512, seed=9)
+    # finite values only (the output check multiplies), still 16 random bits of entropy minus the clamp
+    lin.weight.data = w.float().nan_to_num(0.0, 0.0, 0.0).bfloat16()
+    out = convert(lin, "probe", algo="huffman")
+    text = capsys.readouterr().out
+    assert out is lin and isinstance(out, torch.nn.Linear)
+    assert "ratio" in text and "Fallback to regular nn.Linear" in text

@@ -29,14 +29,14 @@ for cls in (HuffmanWeight, ANSWeight):
         x = torch.randn(1, K, generator=torch.Generator().manual_seed(11)).bfloat16().to(dev)
         y = F.linear(x, mod)
         ref = x.float() @ w.to(dev).float().T
-        torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-3 * max(1.0, ref.abs().max().item()))
+        torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-3)
         print('ok', cls.__name__, M, K, flush=True)
 # a group of two, more tasks than resident wavefronts: units are pulled
 ws = [HuffmanWeight.compress(gaussian_weight(18944, 3584, seed=s)).to(dev) for s in (1, 2)]
 x = torch.randn(1, 3584, generator=torch.Generator().manual_seed(3)).bfloat16().to(dev)
 for y, w in zip(linear_grouped(x, ws), ws):
     ref = x.float() @ w.get_weight().float().T
-    torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-3 * max(1.0, ref.abs().max().item()))
+    torch.testing.assert_close(y.float(), ref, rtol=1e-2, atol=1e-3)
 print('ok group', flush=True)
 """
 

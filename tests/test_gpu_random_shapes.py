@@ -50,7 +50,7 @@ def test_random_shapes(cuda, seed):
         y = torch.nn.functional.linear(x, mod)
         if kind != "bits":
             ref = x.float() @ w.float().T
-            torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL * max(1.0, ref.abs().max().item()), msg=case)
+            torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL, msg=case)
         if it % 3 == 0:
             other = cls.compress(w.flip(0).contiguous()).cuda()
             a, b = linear_grouped(x, [mod, other], [None, None])

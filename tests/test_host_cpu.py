@@ -6,17 +6,29 @@ from bf16_huffman_infer_amd.functional import (ANSWeight, CompressedLinear, Huff
                                                load_compressed_state_dict)
 
 
-def _huffman_weight(M, K):
+def _task_offsets(split_k, M, words_per_task=64):
+    """offsets of a stream with one chunk per row group and equally long tasks (the shapes
+    used here have three steps per split, hence a single chunk)."""
+    off = torch.zeros(split_k, M // 4, 4, dtype=torch.int32)
+    off[:, :, 0] = (torch.arange(split_k * (M // 4), dtype=torch.int32) * words_per_task).view(split_k, M // 4)
+    return off.view(split_k, M), split_k * (M // 4) * words_per_task + 2048
+
+
+def _huffman_weight(M, K, header=(1, 11, 11, 0)):
+    offsets, words = _task_offsets(1, M)
+    code_lengths = torch.zeros(256, dtype=torch.uint8)
+    code_lengths[:4] = torch.tensor(header, dtype=torch.uint8)
     return HuffmanWeight(
-        rem=torch.zeros(1, M, K, dtype=torch.uint8), exp=torch.zeros(4096, dtype=torch.int32),
-        offsets=torch.zeros(1, M, dtype=torch.int32), LUT1=torch.zeros(8192, dtype=torch.uint8),
+        rem=torch.zeros(1, M, K, dtype=torch.uint8), exp=torch.zeros(words, dtype=torch.int32),
+        offsets=offsets, LUT1=torch.zeros(8192, dtype=torch.uint8),
         LUT2=torch.full((256,), 255, dtype=torch.uint8), LUT3=torch.full((256,), 255, dtype=torch.uint8),
-        LUT4=torch.full((256,), 255, dtype=torch.uint8), code_lengths=torch.zeros(256, dtype=torch.uint8))
+        LUT4=torch.full((256,), 255, dtype=torch.uint8), code_lengths=code_lengths)
 
 
 def _ans_weight(M, K):
-    return ANSWeight(rem=torch.zeros(2, M, K // 2, dtype=torch.uint8), exp=torch.zeros(4096, dtype=torch.int32),
-                     offsets=torch.zeros(2, M, dtype=torch.int32), LUT=torch.zeros(256, dtype=torch.int32))
+    offsets, words = _task_offsets(2, M)
+    return ANSWeight(rem=torch.zeros(2, M, K // 2, dtype=torch.uint8), exp=torch.zeros(words, dtype=torch.int32),
+                     offsets=offsets, LUT=torch.zeros(256, dtype=torch.int32))
 
 
 def test_buffer_names_follow_the_reference_modules():
@@ -83,3 +95,63 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
     assert r.returncode != 0
     assert "one GPU" in (r.stderr + r.stdout)
+
+
+def _ans_buffers(layout: str, M=128, K=512):
+    """(rem, exp, offsets, LUT) of a seeded matrix in this package's layout ('wave64') or in the
+    reference package's ('reference'), both written by the numpy models."""
+    import numpy as np
+    from helpers import bits_of, gaussian_weight
+    from oracle import planes, ref_layout, ref_tables, wave64
+    bits = bits_of(gaussian_weight(M, K, seed=2))
+    _, exp = planes.split_bf16(bits)
+    freq, cum, lut = ref_tables.ans_tables(np.bincount(exp.reshape(-1), minlength=256))
+    enc = (wave64.encode_ans(bits, 1, np.asarray(freq), np.asarray(cum)) if layout == "wave64"
+           else ref_layout.encode(bits, 1, "ans", (np.asarray(freq), np.asarray(cum))))
+    return (torch.from_numpy(enc["rem"].copy()), torch.from_numpy(enc["exp"].copy()),
+            torch.from_numpy(enc["offsets"].copy()), torch.from_numpy(np.asarray(lut, dtype=np.int32)))
+
+
+def test_layout_check_accepts_this_packages_buffers_and_rejects_the_references():
+    """A rANS weight saved by the reference package has the same names, dtypes and shapes; only
+    its contents tell it apart, and the kernels must never see it."""
+    from bf16_huffman_infer_amd.functional import check_layout
+    check_layout(ANSWeight(*_ans_buffers("wave64")))
+    with pytest.raises(RuntimeError, match="transcode_reference_weight"):
+        check_layout(ANSWeight(*_ans_buffers("reference")))
+    sd = torch.nn.Sequential(CompressedLinear(ANSWeight(*_ans_buffers("reference")), None)).state_dict()
+    with pytest.raises(RuntimeError, match="transcode_reference_weight"):
+        load_compressed_state_dict(torch.nn.Sequential(torch.nn.Linear(512, 128, bias=False)), sd)
+
+
+def test_layout_check_reads_the_huffman_header():
+    from bf16_huffman_infer_amd.functional import check_layout
+    w = _huffman_weight(128, 384, header=(0, 0, 0, 0))        # not this package's format version
+    with pytest.raises(RuntimeError, match="Huffman tables"):
+        check_layout(w)
+
+
+def test_nibble_window_leaves_room_for_the_escape_nibble():
+    """base + 15 must fit a byte (the decoder adds the base to four nibbles in one 32-bit add)."""
+    from bf16_huffman_infer_amd.functional import NibbleCodec
+    counts = torch.zeros(256, dtype=torch.int64)
+    counts[241:256] = 1000                        # the densest 15-wide window starts at 241
+    counts[3] = 1
+    codec = NibbleCodec(counts)
+    assert codec.base == 240 and codec.has_escapes
+
+
+def test_single_split_weights_may_omit_the_split_dimension():
+    """mv_huffman / mv_ans accept rem [M, N] with offsets [M] (reference functional.py:33-36)."""
+    from bf16_huffman_infer_amd.functional import _promote_single_split
+    rem, off = _promote_single_split(torch.zeros(128, 384, dtype=torch.uint8), torch.zeros(128, dtype=torch.int32))
+    assert tuple(rem.shape) == (1, 128, 384) and tuple(off.shape) == (1, 128)
+    rem3, off2 = torch.zeros(2, 128, 384, dtype=torch.uint8), torch.zeros(2, 128, dtype=torch.int32)
+    assert _promote_single_split(rem3, off2)[0] is rem3 and _promote_single_split(rem3, off2)[1] is off2
+
+
+def test_get_model_size_counts_parameters_and_buffers():
+    from bf16_huffman_infer_amd.utils import get_model_size
+    lin = CompressedLinear(_huffman_weight(128, 384), torch.nn.Parameter(torch.ones(128).bfloat16(), requires_grad=False))
+    want = sum(b.nelement() * b.element_size() for b in lin.weight.buffers()) + 128 * 2
+    assert get_model_size(lin) == want == 128 * 384 + (32 * 64 + 2048) * 4 + 128 * 4 + 8192 + 4 * 256 + 256
