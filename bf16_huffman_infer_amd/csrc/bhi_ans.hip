@@ -120,6 +120,14 @@ extern "C" int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_m
     return bhi_launch_status("gemv_bf16_ans_grouped");
 }
 
+extern "C" int bhi_gemm_bf16_ans(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!weight) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (int rc = launch_mma<AnsCodec>(*weight, X, split_k, Ks, batch, workspace, workspace_bytes, 0, true,
+                                      (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemm_bf16_ans");
+}
+
 extern "C" int bhi_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_words,
                               void* Y, const void* offsets, const void* LUT,
                               int split_k, int M, int Ks, void* stream) {

@@ -193,18 +193,24 @@ struct RowRing {
     // around the ring.  Decided before the loads are issued so that they need not be
     // issued in vain (and so that the compiler cannot sink them behind the decision).
     template <int R>
-    __device__ __forceinline__ bool room() const {
-        const uint32_t top = rhi + R;
+    __device__ __forceinline__ bool room() const { return room_at<R>(rhi); }
+    // The same question for the R rows that start at row `first` >= rhi (a group fetched
+    // further ahead than the next one): positions only advance, so room now is room later.
+    template <int R>
+    __device__ __forceinline__ bool room_at(uint32_t first) const {
+        const uint32_t top = first + R;
         const uint32_t oldest = top > (uint32_t)kRingRows ? (top - kRingRows) << 5 : 0u;
-        return rhi < nrows && ballot(pos < oldest) == 0;
+        return first < nrows && ballot(pos < oldest) == 0;
     }
 
     // The next R rows after the staged ones: one address, immediate offsets.  Rows
     // past the end of the block belong to the next block or to the zero pad that ends the
     // stream; they are loaded, staged, never decoded.
     template <int R>
-    __device__ __forceinline__ void prefetch(uint32_t (&v)[R]) const {
-        const uint32_t* p = bp + (size_t)rhi * kLanes;
+    __device__ __forceinline__ void prefetch(uint32_t (&v)[R]) const { prefetch_at(v, rhi); }
+    template <int R>
+    __device__ __forceinline__ void prefetch_at(uint32_t (&v)[R], uint32_t first) const {
+        const uint32_t* p = bp + (size_t)first * kLanes;
 #pragma unroll
         for (int j = 0; j < R; ++j) v[j] = p[j * kLanes];
     }

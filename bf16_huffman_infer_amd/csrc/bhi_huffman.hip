@@ -127,6 +127,21 @@ extern "C" int bhi_gemv_bf16_huffman_grouped(const bhi_gemv_member* members, int
     return bhi_launch_status("gemv_bf16_huffman_grouped");
 }
 
+extern "C" int bhi_gemm_bf16_huffman(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
+                                     void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!weight) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (int rc = launch_mma<HuffCodec>(*weight, X, split_k, Ks, batch, workspace, workspace_bytes,
+                                       (int64_t)kTableEntries * 4, false, (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemm_bf16_huffman");
+}
+
+extern "C" int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch) {
+    Shape s;
+    if (batch < 1 || batch > kMmaMaxBatch) return bhi_fail(BHI_EBATCH, "the fused matrix product takes 1 to 32 rows of X");
+    if (int rc = check_shape(split_k, M, Ks, kTailPadWords, &s)) return rc;
+    return mma_workspace_bytes(s, batch);
+}
+
 extern "C" int64_t bhi_encode_capacity(int n_steps) {
     if (n_steps < 1) return 0;
     // every lane full of longest codes + every pair escaped + alignment

@@ -1,0 +1,351 @@
+// Fused decode + matrix product for 9..32 rows of X: the weights go from the decoder's
+// registers straight into matrix-core instructions, the compressed bytes are read once
+// and no BF16 weight ever reaches HBM.
+//
+// Stands in for the reference's path above eight rows, `get_weight()` followed by
+// `F.linear` (bf16_huffman_infer/functional.py:405-407, 460-462; decode kernel
+// src/kernel.cu:222-310), which writes the whole BF16 matrix and reads it back through a
+// library GEMM.
+//
+// Shape of the work.  A wavefront decodes the tasks of ONE row group (4 weight rows), as in
+// the GEMV; lane 4b+i holds row i, columns 8b..8b+7 of a step: exactly the A operand of the
+// sixteen 4x4x4 blocks of v_mfma_f32_4x4x4_16b_bf16 (block b = lanes 4b..4b+3, two
+// instructions per step for the two halves of the 8 columns).  The B operand of block b is
+// X[batch 4q+j][the same 4 columns] in lane 4b+j; lane 4b+j then accumulates, for batch
+// quad q, the sums of rows 0..3 for batch 4q+j over column block b (4 registers per quad).
+//
+// X does not come from global memory per wavefront (at 32 rows that would be 8 KB per
+// wavefront and step against 0.7 KB of weights): the block's wavefronts walk the same
+// columns in lockstep, one window of four steps at a time, and the window's slice of X is
+// staged in LDS once per block in the exact order the lanes read it (conflict free,
+// 16 bytes per lane and instruction), double buffered, one barrier per window (a barrier that
+// orders LDS only: the global loads of the next window stay in flight across it).
+//
+// Measured on MI355X, Student-t weights, rotating over 640 MB of clones: 12288x4096 at 16 / 32
+// rows 29.8 / 40.7 us against 56 us for decode-to-BF16 + library GEMM; 4096x12288 (6 K slices)
+// 43 / 61 us against 54-56 us.  Taking the X reads out (wrong results) saves 1.6 / 3.8 us, the
+// barriers 2.8 / 5.7 us; requesting rem bytes, rows and X two windows ahead instead of one was
+// slower (31.7-35.5 us: 128 registers, and nothing was waiting for those loads).  What is left
+// is the decode itself at three to four wavefronts per SIMD -- LDS (two windows of X, rings,
+// table) and 100-128 registers allow no more -- against six in the GEMV.
+//
+// Few row groups (M < 8192) would leave most of the GPU idle, so the tasks of a row group
+// can be dealt to up to 8 blocks (K slices).  Their partial sums meet in a workspace in
+// device memory: every block stores its slice, the last one to arrive at the row block's
+// counter adds the slices in order and writes Y; it leaves the counter at zero.
+#pragma once
+// (included by bhi_task.h users after the static-grid kernels)
+
+namespace bhi {
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kMmaSeg = 4;                   // steps per window
+// wavefronts (row groups) per block: LDS holds two windows of X (8 KB per batch quad) beside
+// the table and the rings; up to 16 rows two 8-wavefront blocks fit a compute unit, above
+// that one block of 16
+constexpr int mma_waves(int Q) { return Q <= 4 ? 8 : 16; }
+constexpr int kMmaMaxBatch = 32;
+constexpr int kMmaMaxSlices = 8;
+constexpr int kMmaSliceBelowGroups = 2048;   // weights with fewer row groups are cut along K
+
+// A block barrier that orders LDS traffic only.  __syncthreads() also waits for every global
+// load in flight (s_waitcnt vmcnt(0)), which would drain the prefetched windows at each barrier.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): this wavefront's LDS writes have landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <int Q>
+struct MmaPolicy {
+    struct Slot { uint2 rem; };
+    struct Piped { int i; };
+    const uint2* rem0;
+    int last;
+    const uint4* xw;          // this lane's 16 bytes of (step 0, quad 0) in the current window
+    f32x4_t acc[Q];
+
+    __device__ __forceinline__ void load(Slot& s, int t) const {
+        t = t < last ? t : last;
+        s.rem = stream_load(rem0 + (size_t)t * kLanes);
+    }
+    __device__ __forceinline__ Piped take(const Slot&, int i, int) const { return Piped{i}; }
+    __device__ __forceinline__ void use(const Piped& p, int, const uint32_t (&w)[4]) {
+        const uint2 a0 = make_uint2(w[0], w[1]), a1 = make_uint2(w[2], w[3]);
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+            const uint4 b = xw[(p.i * Q + q) * kLanes];
+            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4_t, a0), __builtin_bit_cast(short4_t, make_uint2(b.x, b.y)), acc[q], 0, 0, 0);
+            acc[q] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4_t, a1), __builtin_bit_cast(short4_t, make_uint2(b.z, b.w)), acc[q], 0, 0, 0);
+        }
+    }
+};
+
+struct MmaArgs {
+    const uint8_t* rem;
+    const uint32_t* exp;
+    uint16_t* Y;
+    const uint32_t* offsets;
+    const uint32_t* table;
+    const uint8_t* header;
+    const uint16_t* bias;
+    Shape s;
+    int batch;
+    int slices;              // K slices (blocks per row block); divides split_k * nc
+    float* partial;          // [slices][batch][M] when slices > 1
+    uint32_t* counters;      // one per row block, zero between launches
+};
+
+// Workspace layout: the arrival counters first, at a fixed place for every shape (a launch
+// relies on finding them at zero, so no other launch may ever have used those bytes for
+// anything else), then the partial sums.
+constexpr int kMmaCounterBytes = kMmaSliceBelowGroups / 8 * 4;       // sliced launches have fewer row blocks than this
+__host__ __device__ inline long long mma_partial_floats(int M, int batch, int slices) {
+    return slices > 1 ? (long long)slices * batch * M : 0;
+}
+
+template <class Codec, int Q, int NW>
+__global__ __launch_bounds__(NW * kLanes, 4)
+void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
+    constexpr int S = kMmaSeg;
+    constexpr int kWindow = S * Q * kLanes;                   // 16-byte units of one X window
+    constexpr int kThreads = NW * kLanes;
+    constexpr int kPieces = S * Q * 4 * 16;                   // 16-byte pieces of a window: (step, batch row, 8 columns)
+    constexpr int kLoads = (kPieces + kThreads - 1) / kThreads;
+    __shared__ uint32_t rings[NW][kRingWords];
+    __shared__ uint32_t lut[Codec::kTableWords];
+    __shared__ uint4 xbuf[2][kWindow];
+    __shared__ uint32_t is_last;
+
+    const Shape s = a.s;
+    const int lane = threadIdx.x & (kLanes - 1);
+    const int wave = (int)uniform(threadIdx.x / kLanes);
+    const int rb = (int)blockIdx.x / a.slices, ks = (int)blockIdx.x % a.slices;
+    const int g = rb * NW + wave;
+    const int per_group = s.split_k * s.nc;
+    const int tpk = per_group / a.slices;
+    const int kc0 = ks * tpk, kc1 = kc0 + tpk;
+    const int K = s.Ks * s.split_k;
+    const bool variant = Codec::variant(a.header);
+    const int B = a.batch;
+
+    MmaPolicy<Q> pol;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) pol.acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // ---- X staging: piece p of a window = (step i, batch row r = 4q + j, column group b); the
+    // thread that loads it writes it where lane 4b + j will read it
+    static_assert(kLoads <= 2, "two pieces per thread at most");
+    uint4 xg0 = make_uint4(0, 0, 0, 0), xg1 = make_uint4(0, 0, 0, 0);     // (named registers: an array would live in scratch memory)
+    auto piece_load = [&](uint4& dst, int n, int k, int t0, int t_end) __attribute__((always_inline)) {
+        const int p = (int)threadIdx.x + n * kThreads;
+        if (kPieces % kThreads == 0 || p < kPieces) {
+            const int b = p & 15, r = (p >> 4) % (4 * Q), i = p / (64 * Q);
+            const int rr = r < B ? r : B - 1;                     // rows past the batch: any valid row
+            int t = t0 + i;
+            t = t < t_end ? t : t_end - 1;                        // steps past the task: any valid step
+            dst = *(const uint4*)(X + (size_t)rr * K + (size_t)k * s.Ks + (size_t)t * kStepCols + b * kLaneCols);
+        }
+    };
+    auto piece_store = [&](const uint4& src, int n, int par) __attribute__((always_inline)) {
+        const int p = (int)threadIdx.x + n * kThreads;
+        if (kPieces % kThreads == 0 || p < kPieces) {
+            const int b = p & 15, r = (p >> 4) % (4 * Q), i = p / (64 * Q);
+            xbuf[par][(i * Q + (r >> 2)) * kLanes + 4 * b + (r & 3)] = src;
+        }
+    };
+    auto x_load = [&](int k, int t0, int t_end) __attribute__((always_inline)) {       // window starting at step t0 of split k; the task ends at t_end
+        piece_load(xg0, 0, k, t0, t_end);
+        if (kLoads > 1) piece_load(xg1, 1, k, t0, t_end);
+    };
+    auto x_store = [&](int par) __attribute__((always_inline)) {
+        piece_store(xg0, 0, par);
+        if (kLoads > 1) piece_store(xg1, 1, par);
+    };
+
+    typename Codec::Cursor cur;
+    int par = 0;
+    auto walk = [&](auto has_esc) __attribute__((always_inline)) {
+        constexpr bool HAS_ESC = decltype(has_esc)::value;
+        for (int kc = kc0; kc < kc1; ++kc) {
+            const TaskId id = task_of(s, kc);
+            const int ns = id.t1 - id.t0;
+            cur.open(a.exp, task_span(a.offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
+            pol.rem0 = (const uint2*)(a.rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
+            pol.last = ns - 1;
+            typename MmaPolicy<Q>::Slot now[S], next[S];
+#pragma unroll
+            for (int i = 0; i < S; ++i) pol.load(now[i], i);
+            uint32_t first[kPrimeRows];
+            cur.prime_issue(first);
+            if (kc == kc0) {
+                // the table and the first window of X travel with the task's first loads
+                x_load(id.k, id.t0, id.t1);
+                load_table<Codec::kTableWords>(lut, a.table);
+                x_store(0);
+                __syncthreads();
+            }
+            cur.prime_commit(first);
+            cur.start(lut);
+            uint32_t rows[S];
+            bool pending = cur.template room<S>();
+            if (pending) cur.prefetch(rows);
+            const int nseg = (ns + S - 1) / S;
+            for (int seg = 0; seg < nseg; ++seg) {
+                // the window after this one: the task's next, or the next task's first
+                const bool more_here = seg + 1 < nseg, more = more_here || kc + 1 < kc1;
+                if (more_here) {
+                    x_load(id.k, id.t0 + (seg + 1) * S, id.t1);
+                } else if (more) {
+                    const TaskId nx = task_of(s, kc + 1);
+                    x_load(nx.k, nx.t0, nx.t1);
+                }
+                if (pending) cur.commit(rows);
+                pending = cur.template room<S>();
+                if (pending) cur.prefetch(rows);
+#pragma unroll
+                for (int i = 0; i < S; ++i) pol.load(next[i], (seg + 1) * S + i);
+                pol.xw = &xbuf[par][lane];
+                decode_segment<false, HAS_ESC, S>(cur, lut, pol, now, seg * S, ns);
+                if (more) x_store(par ^ 1);
+                lds_barrier();
+                par ^= 1;
+#pragma unroll
+                for (int i = 0; i < S; ++i) now[i] = next[i];
+            }
+        }
+    };
+    if (variant) walk(std::true_type{});
+    else walk(std::false_type{});
+
+    // ---- sums over the 16 column blocks; lane j (< 4) then holds batch 4q + j, rows 0..3
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+#pragma unroll
+        for (int i = 0; i < kGroupRows; ++i) {
+            float v = pol.acc[q][i];
+            v += __shfl_xor(v, 4);
+            v += __shfl_xor(v, 8);
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            pol.acc[q][i] = v;
+        }
+    }
+    if (a.slices == 1) {
+        if (lane < 4) {
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const int batch = 4 * q + lane;
+                if (batch < B) {
+#pragma unroll
+                    for (int i = 0; i < kGroupRows; ++i)
+                        a.Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(pol.acc[q][i], a.bias, kGroupRows * g + i);
+                }
+            }
+        }
+        return;
+    }
+    // ---- K slices: this block's sums go to the workspace with device-scope stores (they
+    // pass the L2 of this die, which the other dies do not see); once they have been
+    // acknowledged the block arrives at its row block's counter.  No cache-wide write-back
+    // or invalidation: with 6144 wavefronts doing one each the launch took 270 us.
+    if (lane < 4) {
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+            const int batch = 4 * q + lane;
+            if (batch < B) {
+                float* dst = a.partial + ((size_t)ks * B + batch) * s.M + kGroupRows * g;
+#pragma unroll
+                for (int i = 0; i < kGroupRows; ++i)
+                    __hip_atomic_store(dst + i, pol.acc[q][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the stores above have completed
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(a.counters + rb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = old == (uint32_t)a.slices - 1;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    // the last block to arrive adds the slices in order (device-scope loads: from memory, not
+    // from a stale line of this die's L2)
+    const int rows_here = kGroupRows * NW;
+    for (int e = threadIdx.x; e < B * rows_here; e += kThreads) {
+        const int batch = e / rows_here, row = rb * rows_here + e % rows_here;
+        float v = 0.f;
+        for (int k = 0; k < a.slices; ++k)
+            v += __hip_atomic_load(a.partial + ((size_t)k * B + batch) * s.M + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        a.Y[(size_t)batch * s.M + row] = finish_output(v, a.bias, row);
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(a.counters + rb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace bhi
+
+// K slices of a launch: enough blocks for the whole GPU where the streams allow it.
+static inline int mma_slices(const bhi::Shape& s, int nw) {
+    using namespace bhi;
+    const int G = s.M / kGroupRows, per_group = s.split_k * s.nc;
+    if (G >= kMmaSliceBelowGroups) return 1;
+    const long long want = 256 * (16 / nw);                  // row blocks x slices: all compute units busy
+    int best = 1;
+    for (int d = 1; d <= kMmaMaxSlices && d <= per_group; ++d)
+        if (per_group % d == 0 && (long long)(G / nw) * best < want) best = d;
+    return best;
+}
+
+static inline int64_t mma_workspace_bytes(const bhi::Shape& s, int batch) {
+    using namespace bhi;
+    const int slices = mma_slices(s, mma_waves((batch + 3) / 4));
+    return slices > 1 ? kMmaCounterBytes + mma_partial_floats(s.M, batch, slices) * 4 : 0;
+}
+
+template <class Codec, int Q>
+static inline void launch_mma_q(const bhi::MmaArgs& a, const uint16_t* x, hipStream_t stream) {
+    using namespace bhi;
+    constexpr int NW = mma_waves(Q);
+    const dim3 grid((unsigned)(a.s.M / (kGroupRows * NW) * a.slices)), block(NW * kLanes);
+    hipLaunchKernelGGL((mma_kernel<Codec, Q, NW>), grid, block, 0, stream, x, a);
+}
+
+template <class Codec>
+static inline int launch_mma(const bhi_gemv_member& m, const void* X, int split_k, int Ks, int batch,
+                             void* workspace, int64_t workspace_bytes, int64_t table_bytes_expected, bool header_is_table,
+                             hipStream_t stream) {
+    using namespace bhi;
+    if (!X || !m.A_rem || !m.A_exp || !m.Y || !m.offsets || !m.table || (!header_is_table && !m.header))
+        return bhi_fail(BHI_EINVAL, "null pointer");
+    if (batch < 1 || batch > kMmaMaxBatch) return bhi_fail(BHI_EBATCH, "the fused matrix product takes 1 to 32 rows of X");
+    if (table_bytes_expected > 0 && m.table_bytes != table_bytes_expected)
+        return bhi_fail(BHI_ELAYOUT, "decode table has the wrong size");
+    Shape s;
+    if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &s)) return rc;
+    const int Q = (batch + 3) / 4, nw = mma_waves(Q);
+    if (m.M % (kGroupRows * nw) != 0) return bhi_fail(BHI_EINVAL, "M must be a multiple of 64");
+    const int slices = mma_slices(s, nw);
+    const int64_t need = mma_workspace_bytes(s, batch);
+    if (slices > 1 && (!workspace || workspace_bytes < need)) return bhi_fail(BHI_EINVAL, "workspace too small: see bhi_gemm_workspace_bytes");
+    MmaArgs a;
+    a.rem = (const uint8_t*)m.A_rem; a.exp = (const uint32_t*)m.A_exp; a.Y = (uint16_t*)m.Y;
+    a.offsets = (const uint32_t*)m.offsets; a.table = (const uint32_t*)m.table;
+    a.header = (const uint8_t*)(header_is_table ? m.table : m.header); a.bias = (const uint16_t*)m.bias;
+    a.s = s; a.batch = batch; a.slices = slices;
+    a.counters = (uint32_t*)workspace;
+    a.partial = (float*)((char*)workspace + kMmaCounterBytes);
+    const uint16_t* x = (const uint16_t*)X;
+    switch (Q) {
+        case 1: launch_mma_q<Codec, 1>(a, x, stream); break;
+        case 2: launch_mma_q<Codec, 2>(a, x, stream); break;
+        case 3: launch_mma_q<Codec, 3>(a, x, stream); break;
+        case 4: launch_mma_q<Codec, 4>(a, x, stream); break;
+        case 5: launch_mma_q<Codec, 5>(a, x, stream); break;
+        case 6: launch_mma_q<Codec, 6>(a, x, stream); break;
+        case 7: launch_mma_q<Codec, 7>(a, x, stream); break;
+        default: launch_mma_q<Codec, 8>(a, x, stream); break;
+    }
+    return 0;
+}

@@ -4,6 +4,7 @@
 // commit / step), the size of its decode table and `variant(header)`, a wave-uniform
 // choice between two instantiations of the walk.
 #pragma once
+#include <type_traits>
 #include "bhi_common.h"
 #include "bhi_host.h"
 
@@ -605,3 +606,5 @@ static inline void launch_decode(const void* A_rem, const void* A_exp, void* Y, 
                        (const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
                        (const uint32_t*)table, (const uint8_t*)header, s);
 }
+
+#include "bhi_mma.h"

@@ -18,8 +18,8 @@ from tqdm import tqdm
 from . import _lib
 from .ans import RANSEncoder
 from .huffman import LUTHuffmanEncoder
-from .ops import (ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemv_bf16_ans,
-                  gemv_bf16_grouped, gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode,
+from .ops import (GEMM_MAX_ROWS, ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemm_bf16,
+                  gemv_bf16_ans, gemv_bf16_grouped, gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode,
                   nibble_decode, nibble_encode, nibble_encode_capacity)
 from .utils import get_block_size_n, split_bf16
 
@@ -632,6 +632,14 @@ def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tens
         output = fused(input)
         if bias is not None:
             output += bias[None, :]
+    elif (input.size(0) <= GEMM_MAX_ROWS and not isinstance(weight, NibbleWeight) and input.dtype == torch.bfloat16
+          and (bias is None or bias.dtype == torch.bfloat16)):
+        # 9..32 rows: decode inside the matrix-core kernel, no BF16 weight in memory
+        split_k, M, N = weight.rem.shape
+        x = input.view(-1, split_k, N)
+        _check_weight_call(weight.rem, weight.exp, x)
+        output = torch.empty((x.size(0), M), dtype=torch.bfloat16, device=x.device)
+        gemm_bf16(weight, x.contiguous(), output, None if bias is None else bias.detach().contiguous())
     else:
         output = F.linear(input, weight.get_weight(), bias)
     return output.unflatten(0, shape[:-1])

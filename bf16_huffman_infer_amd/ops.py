@@ -328,5 +328,82 @@ def gemv_bf16_grouped(weights, X: Tensor, Ys, biases=None) -> None:
         _lib.check(getattr(_lib.load(), entry)(members, len(weights), x_ptr, split_k, Ks, batch, _stream(first.rem)), name)
 
 
+def _fill_member(m, w, Y: Tensor, bias, ref: Tensor) -> bool:
+    """Fills one ``bhi_gemv_member`` from a weight module; returns whether it is a Huffman weight."""
+    huffman = hasattr(w, "LUT1")
+    _, M, _ = _weight_dims(w.rem, w.offsets)
+    m.A_rem = _req(w.rem, torch.uint8, "A_rem", ref)
+    m.A_exp = _req(w.exp, torch.int32, "A_exp", ref)
+    m.exp_words = w.exp.numel()
+    m.Y = _req(Y, torch.bfloat16, "Y", ref)
+    m.offsets = _req(w.offsets, torch.int32, "offsets", ref)
+    if huffman:
+        m.table = _req(w.LUT1, torch.uint8, "LUT1", ref)
+        m.table_bytes = w.LUT1.numel()
+        m.header = _req(w.code_lengths, torch.uint8, "code_lengths", ref)
+    else:
+        m.table = _req(w.LUT, torch.int32, "LUT", ref)
+        m.table_bytes = w.LUT.numel() * 4
+        m.header = None
+    m.M = M
+    if bias is not None:
+        if tuple(bias.shape) != (M,):
+            raise RuntimeError(f"bias must be [{M}], got {tuple(bias.shape)}")
+        m.bias = _req(bias, torch.bfloat16, "bias", ref)
+    return huffman
+
+
+GEMM_MAX_ROWS = 32
+_workspaces = {}          # device -> zero-initialised uint8 tensor; every launch leaves its counters at zero
+
+
+def _gemm_workspace(device: torch.device, nbytes: int) -> Tensor:
+    """The fused matrix product's workspace on ``device``: partial sums of K slices and the
+    arrival counters of their row blocks.  One per device, reused by every call, so calls that
+    overlap on one GPU (different streams) must not share a device's workspace -- as with any
+    library workspace.  Grown by replacement; the old one is kept alive because enqueued
+    launches may still use it."""
+    held = _workspaces.get(device)
+    if held is None or held[-1].numel() < nbytes:
+        fresh = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[device] = (held or []) + [fresh]
+        held = _workspaces[device]
+    return held[-1]
+
+
+def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
+    """``Y = X @ W.T (+ bias)`` for up to 32 rows of ``X`` with ``W`` held compressed
+    (:class:`HuffmanWeight` or :class:`ANSWeight`), decoded inside the matrix-core kernel.
+
+    Takes the place of ``get_weight()`` + ``F.linear`` in the reference's path above eight
+    rows (``functional.py:405-407, 460-462``).  ``X`` bf16 ``[rows, split_k, Ks]``, ``Y`` bf16
+    ``[rows, M]`` written.  Plain function: only enqueues on the current stream (the first call
+    on a device allocates the workspace, so it must not happen under stream capture)."""
+    lib = _lib.load()
+    split_k, M, Ks = _weight_dims(weight.rem, weight.offsets)
+    if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
+        raise RuntimeError(f"X must be [rows, {split_k}, {Ks}], got {tuple(X.shape)}")
+    rows = X.shape[0]
+    if tuple(Y.shape) != (rows, M):
+        raise RuntimeError(f"Y must be [{rows}, {M}], got {tuple(Y.shape)}")
+    member = (_lib.GemvMember * 1)()
+    x_ptr = _req(X, torch.bfloat16, "X", weight.rem)
+    huffman = _fill_member(member[0], weight, Y, bias, weight.rem)
+    name = "gemm_bf16_huffman" if huffman else "gemm_bf16_ans"
+    device = weight.rem.device
+    with torch.cuda.device(device):
+        need = int(lib.bhi_gemm_workspace_bytes(split_k, M, Ks, rows))
+        if need < 0:
+            _lib.check(need, name)
+        held = _workspaces.get(device)
+        if (held is None or held[-1].numel() < need) and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("gemm_bf16: no workspace on this device yet and the stream is capturing; "
+                               "call once outside the capture first")
+        else:
+            ws = _gemm_workspace(device, need)
+            rc = getattr(lib, "bhi_" + name)(member, x_ptr, split_k, Ks, rows, ws.data_ptr(), ws.numel(), _stream(weight.rem))
+    _lib.check(rc, name)
+
+
 def nibble_encode_capacity(n_steps: int) -> int:
     return int(_lib.load().bhi_nibble_encode_capacity(n_steps))

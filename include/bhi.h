@@ -158,6 +158,25 @@ int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, con
 int bhi_gemv_bf16_nibble_grouped(const bhi_gemv_member* members, int n_members, const void* X,
                                  int split_k, int Ks, int batch, void* stream);
 
+/* Fused decode + matrix product for 1..32 rows of X (meant for 9..32; up to 8 the GEMV
+ * entry points are faster): Y = X W^T (+ bias) with the weights going from the decoder's
+ * registers straight into matrix-core instructions.  Replaces the reference's path above
+ * eight rows, huffman_decode / ans_decode to a BF16 matrix followed by a dense GEMM
+ * (functional.py:405-407, 460-462; kernel.cu:510-587, 851-919), which writes and re-reads
+ * 2*M*K bytes per call.  `weight` is one member as the grouped GEMV takes it (Y bf16
+ * [batch, M]; M a multiple of 64).  Weights with fewer than 2048 row groups are cut along K
+ * over several blocks whose partial sums meet in `workspace`: device memory of at least
+ * bhi_gemm_workspace_bytes(...) bytes that was ZERO when first handed to the library and is
+ * otherwise only touched by these entry points (every launch leaves its counters at zero);
+ * launches that may overlap on the GPU must not share a workspace.  It may be NULL when
+ * bhi_gemm_workspace_bytes returns 0. */
+int bhi_gemm_bf16_huffman(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+int bhi_gemm_bf16_ans(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
+                      void* workspace, int64_t workspace_bytes, void* stream);
+/* Workspace bytes a call with these dimensions needs (0: none); negative on a rejected shape. */
+int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch);
+
 /* Readers for weights that were compressed by the reference package itself: same tensors
  * as the reference's huffman_decode / ans_decode ops (kernel.cu:534-587, 878-919) IN THE
  * REFERENCE'S OWN LAYOUT (functional.py:129-242: 64 streams per row, LUT1..4 uint8 [256],

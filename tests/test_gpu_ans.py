@@ -69,8 +69,9 @@ def test_large_batch_falls_back_to_decode_then_gemm(cuda):
     from bf16_huffman_infer_amd.functional import CompressedLinear
     w = gaussian_weight(256, 512, seed=7)
     lin = CompressedLinear(_compress(w), None).cuda()
-    x = torch.randn(12, 512).bfloat16().cuda()
-    torch.testing.assert_close(lin(x).float(), torch.nn.functional.linear(x, w.cuda()).float(), rtol=RTOL, atol=ATOL)
+    for rows in (12, 40):                                    # matrix-core kernel; decode to BF16 + dense GEMM
+        x = torch.randn(rows, 512).bfloat16().cuda()
+        torch.testing.assert_close(lin(x).float(), torch.nn.functional.linear(x, w.cuda()).float(), rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("algo", ["huffman", "ans", "smallest"])

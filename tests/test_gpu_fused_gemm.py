@@ -1,0 +1,70 @@
+"""Fused decode + matrix-core product for 9..32 rows (needs a GPU): against an fp32 matmul of
+the same BF16 operands, and against the decode-then-GEMM path it replaces."""
+import pytest
+import torch
+
+from helpers import gaussian_weight, student_t_weight
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-3
+
+
+def _cls(algo):
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight
+    return {"huffman": HuffmanWeight, "ans": ANSWeight}[algo]
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("rows", [9, 12, 16, 17, 25, 32])
+@pytest.mark.parametrize("make,M,K,n", [(gaussian_weight, 256, 1024, None), (student_t_weight, 128, 512, 2),
+                                        (gaussian_weight, 1024, 4096, None), (student_t_weight, 384, 1536, 4)])
+def test_fused_product_matches_fp32(cuda, algo, rows, make, M, K, n):
+    w = make(M, K, seed=5)
+    mod = (_cls(algo).compress(w) if n is None else _cls(algo).compress_split_n(w, n=n)).cuda()
+    x = torch.randn(rows, K, generator=torch.Generator().manual_seed(rows)).bfloat16().cuda()
+    y = torch.nn.functional.linear(x, mod)
+    assert y.shape == (rows, M) and y.dtype == torch.bfloat16
+    ref = x.float() @ w.cuda().float().T
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+def test_fused_product_with_bias_and_leading_dims(cuda, algo):
+    from bf16_huffman_infer_amd.functional import CompressedLinear
+    w = gaussian_weight(256, 512, seed=7)
+    bias = (torch.randn(256, generator=torch.Generator().manual_seed(1)) * 0.1).bfloat16()
+    lin = CompressedLinear(_cls(algo).compress(w), torch.nn.Parameter(bias, requires_grad=False)).cuda()
+    x = torch.randn(3, 5, 512, generator=torch.Generator().manual_seed(2)).bfloat16().cuda()      # 15 rows
+    y = lin(x)
+    assert y.shape == (3, 5, 256)
+    # the reference's arithmetic: BF16 product, then a BF16 `+= bias`
+    want = (x.float() @ w.cuda().float().T).bfloat16() + bias.cuda()
+    torch.testing.assert_close(y.float(), want.float(), rtol=RTOL, atol=ATOL + 2.0 ** -8 * 0.5)
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("M,K", [(12288, 4096), (4096, 12288)])
+@pytest.mark.parametrize("rows", [16, 32])
+def test_full_size_fallback_shapes(cuda, algo, M, K, rows):
+    """The two layer shapes of the large-batch configuration, Student-t weights: fused product
+    against fp32, and the decoded weight bit for bit."""
+    torch.manual_seed(M + K)
+    w = (torch.distributions.StudentT(3.0).sample((M, K)) * (0.02 / 3 ** 0.5)).bfloat16().cuda()
+    mod = _cls(algo).compress(w).cuda()
+    assert torch.equal(mod.get_weight().view(torch.int16), w.view(torch.int16))
+    x = torch.randn(rows, K, generator=torch.Generator().manual_seed(3)).bfloat16().cuda()
+    y = torch.nn.functional.linear(x, mod)
+    ref = x.float() @ w.float().T
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
+    # twice in a row: the workspace counters are back at zero after every launch
+    y2 = torch.nn.functional.linear(x, mod)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
+def test_more_than_32_rows_still_decode_then_gemm(cuda):
+    w = gaussian_weight(256, 512, seed=7)
+    mod = _cls("huffman").compress(w).cuda()
+    x = torch.randn(40, 512, generator=torch.Generator().manual_seed(2)).bfloat16().cuda()
+    y = torch.nn.functional.linear(x, mod)
+    torch.testing.assert_close(y, torch.nn.functional.linear(x, w.cuda()))
