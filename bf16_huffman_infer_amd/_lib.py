@@ -46,6 +46,8 @@ _SIGNATURES = {
     "bhi_gemm_bf16_huffman": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp, _i64, _vp]),
     "bhi_gemm_bf16_ans": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp, _i64, _vp]),
     "bhi_gemm_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
+    "bhi_gemm_bf16_huffman_static": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp]),
+    "bhi_gemm_static_workspace_bytes": (_i64, []),
     "bhi_reference_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_reference_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
 }

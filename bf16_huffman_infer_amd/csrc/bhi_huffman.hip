@@ -5,6 +5,7 @@
 // one row per 32-lane warp with two private bitstreams per lane and two dependent
 // byte-table reads per exponent; here one 64-lane wavefront walks four rows and one LDS
 // read resolves two exponents.
+#include <mutex>
 #include "bhi_task.h"
 
 namespace bhi {
@@ -134,6 +135,52 @@ extern "C" int bhi_gemm_bf16_huffman(const bhi_gemv_member* weight, const void* 
                                        (int64_t)kTableEntries * 4, false, (hipStream_t)stream)) return rc;
     return bhi_launch_status("gemm_bf16_huffman");
 }
+
+// The workspace of bhi_gemm_bf16_huffman_static: part of the library's image on every GPU
+// that loads it, zero when the image is loaded, and -- like any workspace of these kernels --
+// left with its counters at zero by every launch.
+constexpr int64_t kStaticWorkspaceBytes = (int64_t)kMmaCounterBytes + (2 << 20);
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
+
+// The array's address on the current device.  `scratch` itself is only a host-side handle:
+// each GPU holds its own copy at its own address, looked up once per device.
+static int static_workspace(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static void* known[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return bhi_fail(BHI_EINVAL, "no usable current device");
+    std::lock_guard<std::mutex> hold(lock);
+    if (!known[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return bhi_fail(BHI_EINVAL, "the library's built-in workspace has no address on this device");
+        }
+        known[dev] = p;
+    }
+    *out = known[dev];
+    return 0;
+}
+
+extern "C" int bhi_gemm_bf16_huffman_static(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
+                                            void* stream) {
+    if (!weight) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (batch < 1 || batch > kMmaMaxBatch) return bhi_fail(BHI_EBATCH, "the fused matrix product takes 1 to 32 rows of X");
+    Shape s;
+    if (int rc = check_shape(split_k, weight->M, Ks, weight->exp_words, &s)) return rc;
+    if (mma_workspace_bytes(s, batch) > kStaticWorkspaceBytes)
+        return bhi_fail(BHI_EINVAL, "this product needs more than the 2 MiB of partial sums the built-in workspace holds: "
+                                    "use bhi_gemm_bf16_huffman with a workspace of bhi_gemm_workspace_bytes(...) bytes");
+    void* ws = nullptr;
+    if (int rc = static_workspace(&ws)) return rc;
+    if (int rc = launch_mma<HuffCodec>(*weight, X, split_k, Ks, batch, ws, kStaticWorkspaceBytes,
+                                       (int64_t)kTableEntries * 4, false, (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemm_bf16_huffman_static");
+}
+
+extern "C" int64_t bhi_gemm_static_workspace_bytes(void) { return kStaticWorkspaceBytes; }
 
 extern "C" int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch) {
     Shape s;

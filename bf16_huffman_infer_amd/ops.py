@@ -377,8 +377,10 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
 
     Takes the place of ``get_weight()`` + ``F.linear`` in the reference's path above eight
     rows (``functional.py:405-407, 460-462``).  ``X`` bf16 ``[rows, split_k, Ks]``, ``Y`` bf16
-    ``[rows, M]`` written.  Plain function: only enqueues on the current stream (the first call
-    on a device allocates the workspace, so it must not happen under stream capture)."""
+    ``[rows, M]`` written.  Plain function: only enqueues on the current stream.  The first call
+    on a device allocates the workspace; when that call happens under stream capture, where
+    nothing may be allocated, a Huffman weight goes through the entry point that uses the
+    library's built-in workspace instead."""
     lib = _lib.load()
     split_k, M, Ks = _weight_dims(weight.rem, weight.offsets)
     if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
@@ -397,8 +399,11 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
             _lib.check(need, name)
         held = _workspaces.get(device)
         if (held is None or held[-1].numel() < need) and torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("gemm_bf16: no workspace on this device yet and the stream is capturing; "
-                               "call once outside the capture first")
+            # nothing may be allocated under capture: the library's built-in workspace serves
+            if not huffman or need > int(lib.bhi_gemm_static_workspace_bytes()):
+                raise RuntimeError("gemm_bf16: no workspace on this device yet and the stream is capturing; "
+                                   "call once outside the capture first")
+            rc = lib.bhi_gemm_bf16_huffman_static(member, x_ptr, split_k, Ks, rows, _stream(weight.rem))
         else:
             ws = _gemm_workspace(device, need)
             rc = getattr(lib, "bhi_" + name)(member, x_ptr, split_k, Ks, rows, ws.data_ptr(), ws.numel(), _stream(weight.rem))

@@ -177,6 +177,18 @@ int bhi_gemm_bf16_ans(const bhi_gemv_member* weight, const void* X, int split_k,
 /* Workspace bytes a call with these dimensions needs (0: none); negative on a rejected shape. */
 int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch);
 
+/* bhi_gemm_bf16_huffman without a workspace argument -- no counterpart in the reference.  For
+ * callers that cannot allocate device memory at all (code under stream capture that has no
+ * workspace yet, serving loops and harnesses that forbid it): the partial sums and counters
+ * live in an array inside the library's own device image, bhi_gemm_static_workspace_bytes()
+ * bytes (1 KiB of counters + 2 MiB) on every GPU the library is loaded on.  A product that
+ * needs more (see bhi_gemm_workspace_bytes) is rejected with BHI_EINVAL.  The call allocates
+ * and frees nothing.  All calls on one GPU share the one array: calls that may overlap there
+ * (different streams) race. */
+int bhi_gemm_bf16_huffman_static(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
+                                 void* stream);
+int64_t bhi_gemm_static_workspace_bytes(void);
+
 /* Readers for weights that were compressed by the reference package itself: same tensors
  * as the reference's huffman_decode / ans_decode ops (kernel.cu:534-587, 878-919) IN THE
  * REFERENCE'S OWN LAYOUT (functional.py:129-242: 64 streams per row, LUT1..4 uint8 [256],
