@@ -31,10 +31,26 @@ STD = 0.02
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this script, each scaled by the same counter's reading for the 256 MiB calibration
 # copy below.  Keyed by (algo, batch, launch): "single" = one 18944x3584 matrix, "group" =
-# gate_proj + up_proj in one launch; None where it has not been measured.
-MEASURED_TRAFFIC = {("huffman", 1, "single"): 94_620_000, ("huffman", 1, "group"): 199_860_000,
-                    ("nibble", 1, "single"): 104_700_000, ("nibble", 1, "group"): 223_520_000,
-                    ("ans", 1, "single"): 96_270_000, ("ans", 1, "group"): 205_720_000}
+# gate_proj + up_proj in one launch.  The readings belong to the kernel sources whose digest
+# is recorded with them: when the sources have changed since, `traffic` is reported as null.
+MEASURED_TRAFFIC_SOURCES = "unmeasured"
+MEASURED_TRAFFIC = {}
+
+
+def kernel_sources_digest() -> str:
+    """SHA-256 (first 16 hex digits) over the HIP sources the library is built from."""
+    import hashlib
+    src = os.path.join(ROOT, "bf16_huffman_infer_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(src)):
+        if name.endswith((".h", ".hip")):
+            with open(os.path.join(src, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(key):
+    return MEASURED_TRAFFIC.get(key) if kernel_sources_digest() == MEASURED_TRAFFIC_SOURCES else None
 
 
 def make_weight(M, K, seed, device):
@@ -53,13 +69,55 @@ def gemv_bytes(mod, bs, M, K) -> int:
 
 def build_block(algo, device, copy):
     from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight, NibbleWeight
-    cls = {"huffman": HuffmanWeight, "ans": ANSWeight, "nibble": NibbleWeight}[algo]
+    cls = {"huffman": HuffmanWeight, "ans": ANSWeight, "nibble": NibbleWeight}
     mods = []
     for i, (name, M, K) in enumerate(LAYERS):
         w = make_weight(M, K, 1000 * copy + i, device)
-        mods.append(cls.compress(w).to(device))
+        if algo == "smallest":                      # what convert(..., algo='smallest') keeps: the smaller of the two
+            mods.append(min((HuffmanWeight.compress(w), ANSWeight.compress(w)), key=weight_bytes).to(device))
+        else:
+            mods.append(cls[algo].compress(w).to(device))
         del w
     return mods
+
+
+def sweep(args, device, huffman_blocks):
+    """The same block step at other batches and with the other codecs: GB/s on compressed bytes,
+    fraction of the HBM peak, compressed/raw ratio.  ``smallest`` keeps, per layer, whichever of
+    the Huffman and rANS forms is smaller (gate_proj and up_proj are launched as one group only
+    when they ended up with the same codec)."""
+    import torch.nn.functional as F
+    from bf16_huffman_infer_amd.functional import linear_grouped
+    raw_bytes = sum(M * K * 2 for _, M, K in LAYERS)
+    out = []
+    cases = [("huffman", b) for b in (2, 4, 8)] + [("ans", b) for b in (1, 8)] + [("smallest", b) for b in (1, 8)]
+    built = {"huffman": huffman_blocks}
+    for algo, bs in cases:
+        if algo not in built:
+            built[algo] = [build_block(algo, device, c) for c in range(COPIES)]
+        blocks = built[algo]
+        xs = [torch.randn(bs, K, device=device).bfloat16() for _, _, K in LAYERS]
+        groupable = all(type(b[2]) is type(b[3]) for b in blocks)
+        state = {"i": 0}
+
+        def step():
+            mods = blocks[state["i"] % COPIES]
+            state["i"] += 1
+            F.linear(xs[0], mods[0])
+            F.linear(xs[1], mods[1])
+            if groupable:
+                linear_grouped(xs[2], [mods[2], mods[3]])
+            else:
+                F.linear(xs[2], mods[2])
+                F.linear(xs[3], mods[3])
+            F.linear(xs[4], mods[4])
+        sec = time_launches(step, args.steps, args.warmup, launches_per_graph=COPIES)
+        nbytes = sum(gemv_bytes(m, bs, M, K) for m, (_, M, K) in zip(blocks[0], LAYERS))
+        out.append({"algo": algo, "batch": bs, "ms_per_step": round(sec * 1e3, 5), "GBps": round(nbytes / sec / 1e9, 1),
+                    "frac": round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4),
+                    "compression_ratio": round(sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),
+                    "codecs": sorted({type(m).__name__ for m in blocks[0]})})
+    return out
 
 
 def time_launches(fn, n, warmup, launches_per_graph=1):
@@ -177,6 +235,9 @@ def main():
     ap.add_argument("--algo", default="huffman", choices=["huffman", "ans", "nibble"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-group", action="store_true", help="gate_proj and up_proj as two launches")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the other batches / codecs")
+    ap.add_argument("--no-fallback", action="store_true", help="skip the 16- and 32-row fused matrix product")
+    ap.add_argument("--no-decode", action="store_true", help="skip the 36-layer decoder (tokens/s)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1")
@@ -288,22 +349,41 @@ def main():
         "compressed_bytes_per_step": block_bytes, "compression_ratio": round(
             sum(weight_bytes(m) for m in blocks[0]) / raw_bytes, 4),
         "block_steps_per_s": round(1.0 / sec, 1),
-        # 28 such blocks make one Qwen2.5-7B token (attention, norms, embedding and lm_head not included)
-        "bs1_tokens_per_s_28_blocks": round(1.0 / sec / 28, 1),
+        # DERIVED, not measured: 28 such blocks make one Qwen2.5-7B token (attention, norms, embedding and
+        # lm_head not included); the measured tokens/s of a whole decoder is in "decode"
+        "bs1_tokens_per_s_28_blocks_derived": round(1.0 / sec / 28, 1),
         "us_per_layer": {k: round(v * 1e6, 2) for k, v in per_layer.items()},
         "roofline": {"bound": "hbm", "kernel": f"bhi::gemv_kernel<bhi::{dict(huffman='HuffCodec', ans='AnsCodec', nibble='NibbleCodec')[args.algo]}, {bs}, 4, {2 if args.no_group else 4}> "
                                f"{dom_name}",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.algo, bs, "single" if args.no_group else "group")),
+                     "traffic": measured_traffic((args.algo, bs, "single" if args.no_group else "group")),
                      "bytes_per_launch": dom_bytes, "us_per_launch": round(t_dom * 1e6, 2)},
         # the same kernel launched for one 18944x3584 matrix alone
         "single_launch": {"achieved": round(single_bytes / t_single / 1e9, 1),
                           "frac": round(single_bytes / t_single / 1e9 / HBM_PEAK_GBS, 4),
-                          "traffic": MEASURED_TRAFFIC.get((args.algo, bs, "single")),
+                          "traffic": measured_traffic((args.algo, bs, "single")),
                           "bytes_per_launch": single_bytes, "us_per_launch": round(t_single * 1e6, 2)},
     }
+    out["roofline"]["traffic_from"] = (f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script on kernel sources "
+                                       f"{MEASURED_TRAFFIC_SOURCES}; sources now {kernel_sources_digest()}")
     out["load_only"] = load_only(single_bytes, args, device)
+    del per_layer
+    if not args.no_sweep and args.algo == "huffman" and bs == 1:
+        out["sweep"] = sweep(args, device, blocks)
+    del blocks
+    torch.cuda.empty_cache()
+    if not args.no_fallback:
+        # more than 8 rows of X: the fused decode + matrix-core product beside decode-to-BF16 + dense GEMM
+        from bench_fallback import measure
+        out["fallback"] = measure(device, with_library_gemm=False, steps=max(50, args.steps // 2))
+        torch.cuda.empty_cache()
+    if not args.no_decode:
+        # the tokens/s half of the metric, measured: Qwen3-8B-shaped decoder, 36 layers, algo=smallest,
+        # recorded step, 256 greedy tokens; teacher-forced logits against the raw model
+        import bench_decode
+        out["decode"] = bench_decode.run(bench_decode.parse_args([]))
+        torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

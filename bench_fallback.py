@@ -34,14 +34,12 @@ def student_t(M, K, seed, device):
     return w.bfloat16().to(device)
 
 
-def main():
-    if not torch.cuda.is_available():
-        sys.exit("bench_fallback.py needs a GPU")
-    from bf16_huffman_infer_amd import _lib
+def measure(device, shapes=((12288, 4096), (4096, 12288)), batches=(16, 32), with_library_gemm=True, steps=100):
+    """One dict per (shape, batch); ``with_library_gemm=False`` skips the timings of the decode
+    kernel alone and of the dense GEMM alone."""
     from bf16_huffman_infer_amd.functional import HuffmanWeight
-    _lib.load()
-    device = torch.device("cuda", 0)
-    for (M, K) in ((12288, 4096), (4096, 12288)):
+    results = []
+    for (M, K) in shapes:
         w = student_t(M, K, 7, device)
         mod = HuffmanWeight.compress(w).to(device)
         assert torch.equal(mod.get_weight().view(torch.int16), w.view(torch.int16)), "decode is not lossless"
@@ -53,9 +51,9 @@ def main():
         def decode_only():
             mods[st["i"] % len(mods)].get_weight()
             st["i"] += 1
-        t_dec = time_launches(decode_only, 100, 10, launches_per_graph=len(mods))
+        t_dec = time_launches(decode_only, steps, 10, launches_per_graph=len(mods)) if with_library_gemm else float("nan")
         dec_bytes = weight_bytes(mod) + 2 * M * K
-        for bs in (16, 32):
+        for bs in batches:
             x = torch.randn(bs, K, device=device).bfloat16()
 
             def gemm_only():
@@ -70,12 +68,12 @@ def main():
             def fused():
                 F.linear(x, mods[st["i"] % len(mods)])
                 st["i"] += 1
-            t_gemm = time_launches(gemm_only, 100, 10, launches_per_graph=len(dense))
-            t_all = time_launches(fallback, 100, 10, launches_per_graph=len(mods))
-            t_fused = time_launches(fused, 100, 10, launches_per_graph=len(mods))
+            t_gemm = time_launches(gemm_only, steps, 10, launches_per_graph=len(dense)) if with_library_gemm else float("nan")
+            t_all = time_launches(fallback, steps, 10, launches_per_graph=len(mods))
+            t_fused = time_launches(fused, steps, 10, launches_per_graph=len(mods))
             flops = 2.0 * bs * M * K
             fused_bytes = weight_bytes(mod) + 2 * bs * (M + K)
-            print(json.dumps({
+            results.append({
                 "shape": f"{M}x{K}", "batch": bs, "weights": "Student-t nu=3, std 0.02",
                 "compressed_ratio": round(weight_bytes(mod) / (2 * M * K), 4),
                 "decode_us": round(t_dec * 1e6, 2), "decode_GBps": round(dec_bytes / t_dec / 1e9, 1),
@@ -88,8 +86,18 @@ def main():
                 "fused_frac_of_hbm_peak": round(fused_bytes / t_fused / 8e12, 4),
                 "fused_TFLOPs": round(flops / t_fused / 1e12, 2),
                 "fused_mfma_utilisation": round(flops / t_fused / 1e12 / MFMA_PEAK_TFLOPS, 5),
-            }), flush=True)
+            })
         del mods, dense
+    return results
+
+
+def main():
+    if not torch.cuda.is_available():
+        sys.exit("bench_fallback.py needs a GPU")
+    from bf16_huffman_infer_amd import _lib
+    _lib.load()
+    for r in measure(torch.device("cuda", 0)):
+        print(json.dumps(r), flush=True)
 
 
 if __name__ == "__main__":
