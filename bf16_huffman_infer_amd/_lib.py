@@ -16,7 +16,7 @@ class GemvMember(ctypes.Structure):
     """``bhi_gemv_member`` of include/bhi.h: one weight of a grouped GEMV launch."""
     _fields_ = [("A_rem", _vp), ("A_exp", _vp), ("exp_words", _i64), ("Y", _vp), ("offsets", _vp),
                 ("table", _vp), ("table_bytes", _i64), ("header", _vp), ("bias", _vp), ("M", ctypes.c_int32),
-                ("reserved", ctypes.c_int32)]
+                ("reserved", ctypes.c_int32), ("residual", _vp)]
 
 
 _grouped = (_i32, [ctypes.POINTER(GemvMember), _i32, _vp, _i32, _i32, _i32, _vp])
@@ -43,6 +43,12 @@ _SIGNATURES = {
     "bhi_gemv_bf16_huffman_grouped": _grouped,
     "bhi_gemv_bf16_ans_grouped": _grouped,
     "bhi_gemv_bf16_nibble_grouped": _grouped,
+    "bhi_gemv_bf16_huffman_grouped_x": (_i32, [ctypes.POINTER(GemvMember), _i32, _vp, _i32, _i32, _i32, _i32, _vp,
+                                               ctypes.c_float, _vp]),
+    "bhi_gemv_bf16_ans_grouped_x": (_i32, [ctypes.POINTER(GemvMember), _i32, _vp, _i32, _i32, _i32, _i32, _vp,
+                                           ctypes.c_float, _vp]),
+    "bhi_rms_norm": (_i32, [_vp, _vp, _vp, _i32, _i32, ctypes.c_float, _vp]),
+    "bhi_silu_mul": (_i32, [_vp, _vp, _vp, _i64, _vp]),
     "bhi_gemm_bf16_huffman": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp, _i64, _vp]),
     "bhi_gemm_bf16_ans": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp, _i64, _vp]),
     "bhi_gemm_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),

@@ -16,6 +16,7 @@ constexpr int kAnsInitRows = 2;                 // rows 0, 1 of a lane: its init
 
 struct AnsCodec {
     using Cursor = AnsCursor;
+    static constexpr bool kTransformsX = true;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr bool kPersistent = true;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = kAnsTableWords;
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__) { return false; }
@@ -118,6 +119,14 @@ extern "C" int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_m
                                          int split_k, int Ks, int batch, void* stream) {
     if (int rc = gemv_grouped<AnsCodec>(members, n_members, X, split_k, Ks, batch, 0, true, (hipStream_t)stream)) return rc;
     return bhi_launch_status("gemv_bf16_ans_grouped");
+}
+
+extern "C" int bhi_gemv_bf16_ans_grouped_x(const bhi_gemv_member* members, int n_members, const void* X,
+                                           int split_k, int Ks, int batch, int x_mode, const void* x_aux, float eps,
+                                           void* stream) {
+    if (int rc = gemv_grouped<AnsCodec>(members, n_members, X, split_k, Ks, batch, 0, true, (hipStream_t)stream,
+                                        x_mode, x_aux, eps)) return rc;
+    return bhi_launch_status("gemv_bf16_ans_grouped_x");
 }
 
 extern "C" int bhi_gemm_bf16_ans(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,

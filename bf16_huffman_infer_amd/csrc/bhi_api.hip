@@ -1,7 +1,6 @@
 // Entry points that are not kernels: constants, the chunking rule, error strings.
 #include <stdio.h>
-#include "bhi_common.h"
-#include "bhi_host.h"
+#include "bhi_task.h"
 
 static thread_local char g_err[256] = "";
 
@@ -81,4 +80,59 @@ extern "C" int64_t bhi_stream_read(const void* src, int64_t bytes, int wavefront
         if (int rc = bhi_launch_status("stream_read")) return -(int64_t)(rc > 0 ? rc : -rc);
     }
     return words_per_wave * 4 * wavefronts;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The two layer pieces the GEMV can take in front of its product, as kernels of their own: the
+// unfused form of the same arithmetic (same reduction order, same roundings), used where the
+// fused form does not apply (more than four rows) and as the reference the fused form is
+// tested against bit for bit.
+namespace bhi {
+template <int BS>
+__global__ __launch_bounds__(kBlockThreads) void rms_norm_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ gamma,
+                                                                 uint16_t* __restrict__ out, int K, float eps) {
+    __shared__ float part[kWavesPerBlock * BS];
+    float r[BS];
+    rms_scales_start<BS>(X, K, part);
+    __syncthreads();
+    rms_scales_finish<BS>(part, K, eps, r);
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;          // pair index
+    if (p < K / 2) {
+        const uint32_t g = ((const uint32_t*)gamma)[p];
+#pragma unroll
+        for (int b = 0; b < BS; ++b)
+            ((uint32_t*)out)[(size_t)b * (K / 2) + p] = rms_pair(((const uint32_t*)X)[(size_t)b * (K / 2) + p], r[b], g);
+    }
+}
+
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint32_t* __restrict__ gate, const uint32_t* __restrict__ up,
+                                                       uint32_t* __restrict__ out, long long pairs) {
+    const long long p = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < pairs) out[p] = silu_mul_pair(gate[p], up[p]);
+}
+}  // namespace bhi
+
+extern "C" int bhi_rms_norm(const void* X, const void* gamma, void* out, int rows, int K, float eps, void* stream) {
+    using namespace bhi;
+    if (!X || !gamma || !out) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (rows < 1 || rows > 4 || K < 2 || K % 2 != 0) return bhi_fail(BHI_EINVAL, "rms_norm takes 1 to 4 rows of an even length");
+    const dim3 grid((unsigned)((K / 2 + kBlockThreads - 1) / kBlockThreads)), block(kBlockThreads);
+    const uint16_t *x = (const uint16_t*)X, *g = (const uint16_t*)gamma;
+    uint16_t* o = (uint16_t*)out;
+    switch (rows) {
+        case 1: hipLaunchKernelGGL(rms_norm_kernel<1>, grid, block, 0, (hipStream_t)stream, x, g, o, K, eps); break;
+        case 2: hipLaunchKernelGGL(rms_norm_kernel<2>, grid, block, 0, (hipStream_t)stream, x, g, o, K, eps); break;
+        case 3: hipLaunchKernelGGL(rms_norm_kernel<3>, grid, block, 0, (hipStream_t)stream, x, g, o, K, eps); break;
+        default: hipLaunchKernelGGL(rms_norm_kernel<4>, grid, block, 0, (hipStream_t)stream, x, g, o, K, eps); break;
+    }
+    return bhi_launch_status("rms_norm");
+}
+
+extern "C" int bhi_silu_mul(const void* gate, const void* up, void* out, int64_t n, void* stream) {
+    if (!gate || !up || !out) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (n < 2 || n % 2 != 0) return bhi_fail(BHI_EINVAL, "silu_mul takes an even number of elements");
+    const long long pairs = n / 2;
+    hipLaunchKernelGGL(bhi::silu_mul_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t*)gate, (const uint32_t*)up, (uint32_t*)out, pairs);
+    return bhi_launch_status("silu_mul");
 }

@@ -12,6 +12,7 @@ namespace bhi {
 
 struct HuffCodec {
     using Cursor = HuffCursor;
+    static constexpr bool kTransformsX = true;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr bool kPersistent = true;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = kTableEntries;
     // escaped pairs need the slower walk; the header says whether the matrix has any
@@ -126,6 +127,14 @@ extern "C" int bhi_gemv_bf16_huffman_grouped(const bhi_gemv_member* members, int
     if (int rc = gemv_grouped<HuffCodec>(members, n_members, X, split_k, Ks, batch, (int64_t)kTableEntries * 4, false,
                                          (hipStream_t)stream)) return rc;
     return bhi_launch_status("gemv_bf16_huffman_grouped");
+}
+
+extern "C" int bhi_gemv_bf16_huffman_grouped_x(const bhi_gemv_member* members, int n_members, const void* X,
+                                               int split_k, int Ks, int batch, int x_mode, const void* x_aux, float eps,
+                                               void* stream) {
+    if (int rc = gemv_grouped<HuffCodec>(members, n_members, X, split_k, Ks, batch, (int64_t)kTableEntries * 4, false,
+                                         (hipStream_t)stream, x_mode, x_aux, eps)) return rc;
+    return bhi_launch_status("gemv_bf16_huffman_grouped_x");
 }
 
 extern "C" int bhi_gemm_bf16_huffman(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,

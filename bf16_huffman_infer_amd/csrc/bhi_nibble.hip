@@ -14,6 +14,7 @@ constexpr uint32_t kNibbleEsc = 15;
 
 struct NibbleCodec {
     using Cursor = NibbleCursor;
+    static constexpr bool kTransformsX = false;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr bool kPersistent = false;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = 4;          // base and flags, one 16-byte copy
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ lut) {

@@ -190,15 +190,88 @@ __device__ __forceinline__ void dot_quad4(float& acc, uint32_t x, const uint32_t
         : "+v"(acc) : "v"(x), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
 }
 
+// What the GEMV multiplies the weights with: X as given, or a function of X that the layer in
+// front of the linear would otherwise have to write to memory with a kernel of its own:
+//   kXRms      h = x * rsqrt(mean(x^2) + eps) * gamma      (RMSNorm; gamma bf16 [K])
+//   kXSiluMul  h = silu(gate) * x                          (the SwiGLU product; gate bf16 [batch, K])
+// Both round as the separate kernels of this library do (bhi_rms_norm, bhi_silu_mul), so the
+// fused and the unfused sequence give the same bits.
+enum XMode { kXPlain = 0, kXRms = 1, kXSiluMul = 2 };
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ f32x2_t pair_to_f32(uint32_t p) {
+    return f32x2_t{__uint_as_float(p << 16), __uint_as_float(p & 0xFFFF0000u)};
+}
+__device__ __forceinline__ uint32_t f32_to_pair(f32x2_t v) {           // round to nearest even, both halves
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+// bf16(x * r * gamma), one rounding
+__device__ __forceinline__ uint32_t rms_pair(uint32_t x, float r, uint32_t gamma) {
+    const f32x2_t xf = pair_to_f32(x), gf = pair_to_f32(gamma);
+    return f32_to_pair(f32x2_t{xf.x * r * gf.x, xf.y * r * gf.y});
+}
+// bf16(bf16(silu(g)) * u): the rounding of a BF16 silu followed by a BF16 multiply
+__device__ __forceinline__ uint32_t silu_mul_pair(uint32_t g, uint32_t u) {
+    const f32x2_t gf = pair_to_f32(g), uf = pair_to_f32(u);
+    // g * rcp(1 + 2^(-g * log2 e)): hardware exp2 and reciprocal (one unit in the last place each,
+    // far below the BF16 rounding that follows); a full-precision division here costs more than
+    // the rest of the step
+    const float ex = __builtin_amdgcn_exp2f(gf.x * -1.4426950408889634f), ey = __builtin_amdgcn_exp2f(gf.y * -1.4426950408889634f);
+    const f32x2_t sf = pair_to_f32(f32_to_pair(f32x2_t{gf.x * __builtin_amdgcn_rcpf(1.0f + ex), gf.y * __builtin_amdgcn_rcpf(1.0f + ey)}));
+    return f32_to_pair(f32x2_t{sf.x * uf.x, sf.y * uf.y});
+}
+
+// rsqrt(mean(x^2) + eps) of every batch row, by a whole block: thread t squares the pairs
+// t, t + T, ... of each row, a wavefront adds its lanes' sums by xor-shuffles, the
+// wavefronts' sums meet in `part` ([waves][BS] floats in LDS) and are added in order after
+// the caller's next barrier (rms_scales_finish).  The same code serves the stand-alone
+// RMSNorm kernel, which is what makes fused and unfused results identical.
 template <int BS>
+__device__ __forceinline__ void rms_scales_start(const uint16_t* __restrict__ X, int K, float* part) {
+    const int lane = threadIdx.x & (kLanes - 1), wave = threadIdx.x / kLanes;
+    float sq[BS];
+#pragma unroll
+    for (int b = 0; b < BS; ++b) sq[b] = 0.f;
+    for (int p = threadIdx.x; p < K / 2; p += blockDim.x) {
+#pragma unroll
+        for (int b = 0; b < BS; ++b) {
+            const f32x2_t v = pair_to_f32(((const uint32_t*)X)[(size_t)b * (K / 2) + p]);
+            sq[b] += v.x * v.x;
+            sq[b] += v.y * v.y;
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < BS; ++b) {
+        float v = sq[b];
+        for (int o = 1; o < kLanes; o <<= 1) v += __shfl_xor(v, o);
+        if (lane == 0) part[wave * BS + b] = v;
+    }
+}
+template <int BS>
+__device__ __forceinline__ void rms_scales_finish(const float* part, int K, float eps, float (&r)[BS]) {
+    const int waves = blockDim.x / kLanes;
+#pragma unroll
+    for (int b = 0; b < BS; ++b) {
+        float v = 0.f;
+        for (int w = 0; w < waves; ++w) v += part[w * BS + b];
+        r[b] = 1.0f / sqrtf(v / (float)K + eps);
+    }
+}
+
+template <int BS, int XM = kXPlain>
 struct DotPolicy {
+    static_assert(XM == kXPlain || BS <= 4, "transformed X is kept in the segment's operand set: batch 1..4");
     static constexpr int NSET = BS <= 4 ? 1 : 2;            // batch rows in sets of four
     static constexpr bool PIPED = BS > 4;
     static constexpr int XAHEAD = BS > 6 ? 1 : 2;            // 92 registers at batch 8: five wavefronts per SIMD
-    struct Slot { uint2 rem; uint4 x; };                     // x: the lane's X pair of batch rows 0..3
-    struct Piped { uint4 x; int i, t; };
+    struct Slot { uint2 rem; uint4 x; uint4 a; };            // x: the lane's X pair of batch rows 0..3; a: gamma or gate pairs
+    struct Piped { uint4 x, a; int i, t; };
     const uint2* rem0;
     const uint32_t* xq0;     // this lane's X pair of batch row 0, first step of the task
+    const uint32_t* aq0;     // the same position in gamma (kXRms) or in gate row 0 (kXSiluMul)
+    float rs[BS <= 4 ? BS : 1];   // kXRms: the rows' scales
     int xrow;                // distance between batch rows of X, in pairs
     int last;
     uint4 xr[XAHEAD][NSET];  // batch 5..8: the pairs of the next XAHEAD steps
@@ -224,26 +297,33 @@ struct DotPolicy {
             for (int i = 0; i < XAHEAD; ++i) xload(xr[i], i);
         }
     }
-    __device__ __forceinline__ void load(Slot& s, int t) const { load_at(s, rem0, xq0, last, t); }
-    // step t (clamped to last_) of the task whose first step sits at r0 / x0
-    __device__ __forceinline__ void load_at(Slot& s, const uint2* r0, const uint32_t* x0, int last_, int t) const {
+    __device__ __forceinline__ void load(Slot& s, int t) const { load_at(s, rem0, xq0, last, t, aq0); }
+    // step t (clamped to last_) of the task whose first step sits at r0 / x0 (/ a0)
+    __device__ __forceinline__ void load_at(Slot& s, const uint2* r0, const uint32_t* x0, int last_, int t,
+                                            const uint32_t* a0 = nullptr) const {
         t = t < last_ ? t : last_;
         s.rem = stream_load(r0 + (size_t)t * kLanes);
         if (!PIPED) xpairs<0>(s.x, x0 + (size_t)t * (kStepCols / 2));
+        if (XM == kXRms) s.a.x = a0[(size_t)t * (kStepCols / 2)];
+        if (XM == kXSiluMul) xpairs<0>(s.a, a0 + (size_t)t * (kStepCols / 2));
     }
     template <int S>
     __device__ __forceinline__ void load_full(Slot (&s)[S], int t0) const {
         const uint2* pr = rem0 + (size_t)t0 * kLanes;
         const uint32_t* pq = xq0 + (size_t)t0 * (kStepCols / 2);
+        const uint32_t* pa = aq0 + (size_t)t0 * (kStepCols / 2);
 #pragma unroll
         for (int i = 0; i < S; ++i) {
             s[i].rem = stream_load(pr + i * kLanes);
             if (!PIPED) xpairs<0>(s[i].x, pq + i * (kStepCols / 2));
+            if (XM == kXRms) s[i].a.x = pa[i * (kStepCols / 2)];
+            if (XM == kXSiluMul) xpairs<0>(s[i].a, pa + i * (kStepCols / 2));
         }
     }
     __device__ __forceinline__ Piped take(const Slot& s, int i, int t) const {
         Piped p;
         if (!PIPED) p.x = s.x;
+        if (XM != kXPlain) p.a = s.a;
         p.i = i;
         p.t = t;
         return p;
@@ -252,7 +332,16 @@ struct DotPolicy {
 #pragma unroll
         for (int q = 0; q < NSET; ++q) {
             const uint4 xs = PIPED ? xr[s.i % XAHEAD][q] : s.x;
-            const uint32_t xb[4] = {xs.x, xs.y, xs.z, xs.w};
+            uint32_t xb[4] = {xs.x, xs.y, xs.z, xs.w};
+            if (XM == kXRms) {
+#pragma unroll
+                for (int j = 0; j < BS && j < 4; ++j) xb[j] = rms_pair(xb[j], rs[j], s.a.x);
+            }
+            if (XM == kXSiluMul) {
+                const uint32_t gb[4] = {s.a.x, s.a.y, s.a.z, s.a.w};
+#pragma unroll
+                for (int j = 0; j < BS && j < 4; ++j) xb[j] = silu_mul_pair(gb[j], xb[j]);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (4 * q + j < BS) dot_quad4(dot[4 * q + j], xb[j], w);
@@ -353,28 +442,34 @@ struct Member {
     const uint32_t* table;
     const uint8_t* header;
     const uint16_t* bias;    // bf16 [M] or null
+    const uint16_t* residual;   // bf16 [batch, M] or null: added last, as a separate BF16 `y + residual` would
     Shape s;
     int first_block;         // this member's blocks are [first_block, next member's first_block)
 };
 struct Group {
     int n;
     Member m[kMaxMembers];
+    const uint16_t* xaux;    // gamma (kXRms) or gate (kXSiluMul)
+    float eps;               // kXRms
 };
 
 // The sum rounded to BF16; with a bias, that BF16 value plus the bias, rounded again (what a
 // separate BF16 `output += bias` after the product gives).
-__device__ __forceinline__ uint16_t finish_output(float sum, const uint16_t* __restrict__ bias, int row) {
+__device__ __forceinline__ uint16_t finish_output(float sum, const uint16_t* __restrict__ bias, int row,
+                                                  const uint16_t* __restrict__ residual_row = nullptr) {
     uint16_t y = f32_to_bf16_rne(sum);
     if (bias) y = f32_to_bf16_rne(__uint_as_float((uint32_t)y << 16) + __uint_as_float((uint32_t)bias[row] << 16));
+    if (residual_row) y = f32_to_bf16_rne(__uint_as_float((uint32_t)y << 16) + __uint_as_float((uint32_t)residual_row[row] << 16));
     return y;
 }
 
-template <class Codec, int BS, int NW, int S>
+template <class Codec, int BS, int NW, int S, int XM = kXPlain>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
 void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     // The partial sums reuse the rings once every task of the block is done.
     __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
+    __shared__ float rms_part[XM == kXRms ? NW * BS : 1];
     int member = 0;
 #pragma unroll
     for (int i = 1; i < kMaxMembers; ++i)
@@ -387,6 +482,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     const uint32_t* __restrict__ table = mb.table;
     const uint8_t* __restrict__ header = mb.header;
     const uint16_t* __restrict__ bias = mb.bias;
+    const uint16_t* __restrict__ residual = mb.residual;
     const Shape s = mb.s;
     const int block = (int)blockIdx.x - mb.first_block;
     // P wavefronts share one row group; a block holds NW / P row groups
@@ -414,13 +510,23 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     const int K = s.Ks * s.split_k;
     const bool variant = Codec::variant(header);
 
-    DotPolicy<BS> pol;
-    constexpr int NSET = DotPolicy<BS>::NSET;
+    DotPolicy<BS, XM> pol;
+    constexpr int NSET = DotPolicy<BS, XM>::NSET;
 #pragma unroll
     for (int q = 0; q < NSET; ++q) pol.acc[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 8; ++j) pol.dot[j] = 0.f;
     pol.xrow = K / 2;
+    // RMSNorm in front of the product: every wavefront of the block squares its share of X
+    // (also one without a task) behind its first loads; the sums are complete behind the
+    // barrier that ends the table copy
+    auto stage_all = [&]() {
+        if (!staged) {
+            if constexpr (XM == kXRms) rms_scales_start<BS>(X, K, rms_part);
+            stage_table();
+            if constexpr (XM == kXRms) rms_scales_finish<BS>(rms_part, K, grp.eps, pol.rs);
+        }
+    };
 
     if (active) {
         for (int kc = p; kc < per_group; kc += P) {
@@ -429,9 +535,11 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
             cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
             pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
             pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
+            pol.aq0 = XM == kXPlain ? nullptr
+                                    : (const uint32_t*)(grp.xaux + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
-            if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_table);
-            else run_task<false, S>(cur, lut, pol, id.t1 - id.t0, stage_table);
+            if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
+            else run_task<false, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
         }
         pol.fold();
         // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
@@ -448,7 +556,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
             }
         }
     }
-    stage_table();
+    stage_all();
     if (P == 1) {
         // one wavefront per row group: its sums are final
         if (active && lane < 4) {
@@ -458,7 +566,8 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
                 if (batch < BS) {
 #pragma unroll
                     for (int i = 0; i < kGroupRows; ++i)
-                        Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(pol.acc[q][i], bias, kGroupRows * g + i);
+                        Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(pol.acc[q][i], bias, kGroupRows * g + i,
+                                                                                    residual ? residual + (size_t)batch * s.M : nullptr);
                 }
             }
         }
@@ -482,7 +591,8 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
                 for (int i = 0; i < kGroupRows; ++i) {
                     float a = 0.f;
                     for (int w = 0; w < P; ++w) a += ((const float*)rings[rg * P + w])[(q * kGroupRows + i) * 4 + lane];
-                    Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(a, bias, kGroupRows * g + i);
+                    Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(a, bias, kGroupRows * g + i,
+                                                                                residual ? residual + (size_t)batch * s.M : nullptr);
                 }
             }
         }
@@ -533,10 +643,31 @@ static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks,
         hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegShort>), grid, block, 0, stream, (const uint16_t*)X, grp);
 }
 
+// Launches with a transformed X (kXRms, kXSiluMul): batch 1..4, short segments.
+template <class Codec, int XM>
+static inline void launch_gemv_x(int batch, const void* X, const bhi::Group& grp, int blocks, hipStream_t stream) {
+    using namespace bhi;
+    const dim3 grid((unsigned)blocks), block(kWavesPerBlock * kLanes);
+    const uint16_t* x = (const uint16_t*)X;
+    switch (batch) {
+        case 1: hipLaunchKernelGGL((gemv_kernel<Codec, 1, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
+        case 2: hipLaunchKernelGGL((gemv_kernel<Codec, 2, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
+        case 3: hipLaunchKernelGGL((gemv_kernel<Codec, 3, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
+        default: hipLaunchKernelGGL((gemv_kernel<Codec, 4, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
+    }
+}
+
 template <class Codec>
-static inline void launch_gemv_batch(int batch, const void* X, const bhi::Group& grp, int blocks, hipStream_t st) {
+static inline void launch_gemv_batch(int batch, const void* X, const bhi::Group& grp, int blocks, hipStream_t st,
+                                     int x_mode = bhi::kXPlain) {
+    if constexpr (Codec::kTransformsX) {
+        if (x_mode == bhi::kXRms) return launch_gemv_x<Codec, bhi::kXRms>(batch, X, grp, blocks, st);
+        if (x_mode == bhi::kXSiluMul) return launch_gemv_x<Codec, bhi::kXSiluMul>(batch, X, grp, blocks, st);
+    }
     if constexpr (Codec::kPersistent) {
-        if (try_launch_persist<Codec>(batch, X, grp, st)) return;
+        bool plain = true;
+        for (int i = 0; i < grp.n; ++i) plain = plain && !grp.m[i].residual;
+        if (plain && try_launch_persist<Codec>(batch, X, grp, st)) return;
     }
     switch (batch) {
         case 1: launch_gemv<Codec, 1>(X, grp, blocks, st); break;
@@ -558,24 +689,33 @@ static inline void launch_gemv_batch(int batch, const void* A_rem, const void* A
     bhi::Group grp = {};
     grp.n = 1;
     grp.m[0] = bhi::Member{(const uint8_t*)A_rem, (const uint32_t*)A_exp, (uint16_t*)Y, (const uint32_t*)offsets,
-                           (const uint32_t*)table, (const uint8_t*)header, nullptr, s, 0};
+                           (const uint32_t*)table, (const uint8_t*)header, nullptr, nullptr, s, 0};
     launch_gemv_batch<Codec>(batch, X, grp, gemv_blocks(s), st);
 }
 
-static_assert(sizeof(bhi_gemv_member) == 80, "bindings mirror this struct field by field");
+static_assert(sizeof(bhi_gemv_member) == 88, "bindings mirror this struct field by field");
 
 // The grouped entry points: members of one codec that share X, split_k and Ks.
 // `table_bytes_expected` > 0 checks every member's table size (Huffman).
 template <class Codec>
 static inline int gemv_grouped(const bhi_gemv_member* members, int n_members, const void* X, int split_k, int Ks,
-                               int batch, int64_t table_bytes_expected, bool header_is_table, hipStream_t st) {
+                               int batch, int64_t table_bytes_expected, bool header_is_table, hipStream_t st,
+                               int x_mode = bhi::kXPlain, const void* x_aux = nullptr, float eps = 0.f) {
     using namespace bhi;
     if (!members || !X) return bhi_fail(BHI_EINVAL, "null pointer");
     if (n_members < 1 || n_members > kMaxMembers) return bhi_fail(BHI_EINVAL, "a group has 1 to 4 members");
     if (batch < 1) return bhi_fail(BHI_EINVAL, "batch must be >= 1");
     if (batch > kMaxBatch) return bhi_fail(BHI_EBATCH, "fused GEMV supports batch <= 8");
+    if (x_mode != kXPlain) {
+        if (x_mode != kXRms && x_mode != kXSiluMul) return bhi_fail(BHI_EINVAL, "unknown X transform");
+        if (!Codec::kTransformsX) return bhi_fail(BHI_EINVAL, "this codec's kernels take X as it is");
+        if (!x_aux) return bhi_fail(BHI_EINVAL, "the X transform needs its second operand (gamma or gate)");
+        if (batch > 4) return bhi_fail(BHI_EBATCH, "a transformed X is fused for batch <= 4");
+    }
     Group grp = {};
     grp.n = n_members;
+    grp.xaux = (const uint16_t*)x_aux;
+    grp.eps = eps;
     long long blocks = 0;
     for (int i = 0; i < n_members; ++i) {
         const bhi_gemv_member& m = members[i];
@@ -587,11 +727,11 @@ static inline int gemv_grouped(const bhi_gemv_member* members, int n_members, co
         if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &s)) return rc;
         grp.m[i] = Member{(const uint8_t*)m.A_rem, (const uint32_t*)m.A_exp, (uint16_t*)m.Y, (const uint32_t*)m.offsets,
                           (const uint32_t*)m.table, (const uint8_t*)(header_is_table ? m.table : m.header),
-                          (const uint16_t*)m.bias, s, (int)blocks};
+                          (const uint16_t*)m.bias, (const uint16_t*)m.residual, s, (int)blocks};
         blocks += gemv_blocks(s);
     }
     if (blocks > 0x7FFFFFFFll) return bhi_fail(BHI_EINVAL, "group too large for one launch");
-    launch_gemv_batch<Codec>(batch, X, grp, (int)blocks, st);
+    launch_gemv_batch<Codec>(batch, X, grp, (int)blocks, st, x_mode);
     return 0;
 }
 

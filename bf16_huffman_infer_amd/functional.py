@@ -18,6 +18,7 @@ from tqdm import tqdm
 from . import _lib
 from .ans import RANSEncoder
 from .huffman import LUTHuffmanEncoder
+from . import ops as _ops
 from .ops import (GEMM_MAX_ROWS, ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemm_bf16,
                   gemv_bf16_ans, gemv_bf16_grouped, gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode,
                   nibble_decode, nibble_encode, nibble_encode_capacity)
@@ -399,28 +400,60 @@ class CompressedLinear(nn.Module):
         return F.linear(input, self.weight, self.bias)
 
 
-def linear_grouped(input: Tensor, weights, biases=None) -> list:
-    """``[F.linear(input, w, b) for w, b in zip(weights, biases)]`` in ONE launch.
+def linear_grouped(input: Tensor, weights, biases=None, *, residuals=None, input_norm=None, input_gate=None,
+                   outs=None) -> list:
+    """``[F.linear(h, w, b) (+ r) for w, b, r in zip(weights, biases, residuals)]`` in ONE launch, where
+    ``h`` is ``input``, or -- so that the layer in front of the linears needs no kernel of its own --
+
+    * ``input_norm=(gamma, eps)``: ``h = rms_norm(input) * gamma`` (RMSNorm in front of q/k/v or gate/up),
+    * ``input_gate=gate``: ``h = silu(gate) * input`` (the SwiGLU product in front of down_proj).
 
     ``weights`` are up to four compressed weights of one class with the same
     ``in_features`` split (``rem.shape[0]`` and ``rem.shape[2]``); ``input`` has at most
-    8 rows after flattening.  This is what the q/k/v (or gate/up) projections of a
+    8 rows after flattening.  ``residuals[i]`` (shaped like output ``i``) is added last, as a
+    separate BF16 addition would; ``outs[i]`` (bf16 ``[rows, M_i]``, contiguous -- a column slice of a
+    one-row buffer qualifies) receives output ``i`` instead of a new tensor.  This is what the q/k/v (or gate/up) projections of a
     decoder layer need: the reference overlaps them on parallel streams
-    (``cudastream_utils.py:8-47``), here they are one grid.
+    (``cudastream_utils.py:8-47``), here they are one grid.  Up to 4 rows (Huffman, rANS) the
+    norm / gate product happens inside the kernel; otherwise it runs as this package's own
+    elementwise kernel first -- the same arithmetic, the same bits.
     """
     assert input.dim() >= 2, input
+    assert input_norm is None or input_gate is None, "one transform of the input at a time"
     shape = input.shape
     x = input.flatten(0, -2)
     if x.size(0) > MAX_FUSED_BATCH:
         raise RuntimeError(f'linear_grouped takes at most {MAX_FUSED_BATCH} rows, got {x.size(0)}')
     first = weights[0]
     split_k, _, N = first.rem.shape
+    mode, aux, eps = _ops.X_PLAIN, None, 0.0
+    if input_norm is not None or input_gate is not None:
+        fusable = x.size(0) <= _ops.X_TRANSFORM_MAX_ROWS and not isinstance(first, NibbleWeight)
+        if input_norm is not None:
+            gamma, eps = input_norm
+            gamma = gamma.detach()
+            if fusable:
+                mode, aux = _ops.X_RMS, gamma.contiguous()
+            else:
+                x = _ops.rms_norm(x, gamma, eps)
+        else:
+            gate = input_gate.flatten(0, -2)
+            assert gate.shape == x.shape, (gate.shape, x.shape)
+            if fusable:
+                mode, aux = _ops.X_SILU_MUL, gate.contiguous()
+            else:
+                x = _ops.silu_mul(gate, x)
     x = x.view(-1, split_k, N)
     _check_weight_call(first.rem, first.exp, x)
-    ys = [torch.empty((x.size(0), w.rem.shape[1]), dtype=torch.bfloat16, device=x.device) for w in weights]
+    if outs is not None:
+        ys = [o.view(x.size(0), w.rem.shape[1]) for o, w in zip(outs, weights)]
+    else:
+        ys = [torch.empty((x.size(0), w.rem.shape[1]), dtype=torch.bfloat16, device=x.device) for w in weights]
     if biases is not None:
         biases = [None if b is None else b.detach().contiguous() for b in biases]
-    gemv_bf16_grouped(weights, x.contiguous(), ys, biases)
+    if residuals is not None:
+        residuals = [None if r is None else r.detach().reshape(x.size(0), -1).contiguous() for r in residuals]
+    gemv_bf16_grouped(weights, x.contiguous(), ys, biases, residuals, mode, aux, float(eps))
     return [y.unflatten(0, shape[:-1]) for y in ys]
 
 

@@ -269,27 +269,37 @@ def nibble_decode(A_rem: Tensor, A_exp: Tensor, Y: Tensor, offsets: Tensor, LUT:
     torch.ops.bf16_huffman_infer.nibble_decode.default(A_rem, A_exp, Y, offsets, LUT)
 
 
-def gemv_bf16_grouped(weights, X: Tensor, Ys, biases=None) -> None:
+X_PLAIN, X_RMS, X_SILU_MUL = 0, 1, 2
+X_TRANSFORM_MAX_ROWS = 4
+
+
+def gemv_bf16_grouped(weights, X: Tensor, Ys, biases=None, residuals=None, x_mode: int = X_PLAIN, x_aux=None,
+                      eps: float = 0.0) -> None:
     """One launch for up to four compressed weights that multiply the same ``X``.
 
     ``weights`` are weight modules of ONE class (:class:`HuffmanWeight`, :class:`ANSWeight`
     or :class:`NibbleWeight`: anything with ``rem, exp, offsets`` and ``LUT1, code_lengths``
     or ``LUT``) with equal ``split_k`` and ``Ks``; ``X`` is bf16 ``[batch, split_k, Ks]``,
     ``Ys[i]`` bf16 ``[batch, M_i]`` is written; ``biases[i]`` (bf16 ``[M_i]`` or None) is added
-    as the reference's separate ``output += bias`` would (``functional.py:403-404``).  Not an op of the reference: it stands in
-    for its q/k/v streams (``cudastream_utils.py:8-47``).  Plain function, not registered
-    with the dispatcher; like the ops it only enqueues on the current stream.
+    as the reference's separate ``output += bias`` would (``functional.py:403-404``), then
+    ``residuals[i]`` (bf16 ``[batch, M_i]`` or None) as a separate BF16 addition would.
+    ``x_mode`` makes the kernel multiply with a function of ``X`` (batch <= 4, Huffman and
+    rANS): ``X_RMS`` -- RMSNorm of ``X`` with ``x_aux`` = gamma bf16 ``[split_k*Ks]`` and
+    ``eps``; ``X_SILU_MUL`` -- ``silu(x_aux) * X`` with ``x_aux`` = gate, shaped like ``X``.
+    Not an op of the reference: it stands in for its q/k/v streams
+    (``cudastream_utils.py:8-47``).  Plain function, not registered with the dispatcher; like
+    the ops it only enqueues on the current stream.
     """
     if not 1 <= len(weights) <= 4 or len(weights) != len(Ys):
         raise RuntimeError("a group has 1 to 4 weights and one output per weight")
     first = weights[0]
     huffman = hasattr(first, "LUT1")
     if huffman:
-        entry, name = "bhi_gemv_bf16_huffman_grouped", "gemv_bf16_huffman_grouped"
+        entry = "gemv_bf16_huffman_grouped"
     elif int(getattr(first, "MAGIC", 0)) != 0:
-        entry, name = "bhi_gemv_bf16_nibble_grouped", "gemv_bf16_nibble_grouped"
+        entry = "gemv_bf16_nibble_grouped"
     else:
-        entry, name = "bhi_gemv_bf16_ans_grouped", "gemv_bf16_ans_grouped"
+        entry = "gemv_bf16_ans_grouped"
     split_k, _, Ks = _weight_dims(first.rem, first.offsets)
     if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
         raise RuntimeError(f"X must be [batch, {split_k}, {Ks}], got {tuple(X.shape)}")
@@ -298,7 +308,9 @@ def gemv_bf16_grouped(weights, X: Tensor, Ys, biases=None) -> None:
     members = (_lib.GemvMember * len(weights))()
     if biases is None:
         biases = [None] * len(weights)
-    for m, w, Y, b in zip(members, weights, Ys, biases):
+    if residuals is None:
+        residuals = [None] * len(weights)
+    for m, w, Y, b, r in zip(members, weights, Ys, biases, residuals):
         if type(w) is not type(first):
             raise RuntimeError("the weights of a group must use one codec")
         sk, M, ks = _weight_dims(w.rem, w.offsets)
@@ -306,26 +318,54 @@ def gemv_bf16_grouped(weights, X: Tensor, Ys, biases=None) -> None:
             raise RuntimeError("the weights of a group must share split_k and Ks")
         if tuple(Y.shape) != (batch, M):
             raise RuntimeError(f"Y must be [{batch}, {M}], got {tuple(Y.shape)}")
-        m.A_rem = _req(w.rem, torch.uint8, "A_rem", first.rem)
-        m.A_exp = _req(w.exp, torch.int32, "A_exp", first.rem)
-        m.exp_words = w.exp.numel()
-        m.Y = _req(Y, torch.bfloat16, "Y", first.rem)
-        m.offsets = _req(w.offsets, torch.int32, "offsets", first.rem)
-        if huffman:
-            m.table = _req(w.LUT1, torch.uint8, "LUT1", first.rem)
-            m.table_bytes = w.LUT1.numel()
-            m.header = _req(w.code_lengths, torch.uint8, "code_lengths", first.rem)
-        else:
-            m.table = _req(w.LUT, torch.int32, "LUT", first.rem)
-            m.table_bytes = w.LUT.numel() * 4
-            m.header = None
-        m.M = M
-        if b is not None:
-            if tuple(b.shape) != (M,):
-                raise RuntimeError(f"bias must be [{M}], got {tuple(b.shape)}")
-            m.bias = _req(b, torch.bfloat16, "bias", first.rem)
+        _fill_member(m, w, Y, b, first.rem)
+        if r is not None:
+            if tuple(r.shape) != (batch, M):
+                raise RuntimeError(f"residual must be [{batch}, {M}], got {tuple(r.shape)}")
+            m.residual = _req(r, torch.bfloat16, "residual", first.rem)
+    lib = _lib.load()
     with torch.cuda.device(first.rem.device):
-        _lib.check(getattr(_lib.load(), entry)(members, len(weights), x_ptr, split_k, Ks, batch, _stream(first.rem)), name)
+        if x_mode == X_PLAIN:
+            rc = getattr(lib, "bhi_" + entry)(members, len(weights), x_ptr, split_k, Ks, batch, _stream(first.rem))
+        else:
+            if entry == "gemv_bf16_nibble_grouped":
+                raise RuntimeError("the nibble codec's kernels take X as it is")
+            want = (split_k * Ks,) if x_mode == X_RMS else (batch, split_k * Ks)
+            if x_aux is None or x_aux.numel() != want[-1] * (1 if x_mode == X_RMS else batch):
+                raise RuntimeError(f"x_aux must hold {want} values")
+            entry += "_x"
+            rc = getattr(lib, "bhi_" + entry)(members, len(weights), x_ptr, split_k, Ks, batch, int(x_mode),
+                                              _req(x_aux, torch.bfloat16, "x_aux", first.rem), float(eps), _stream(first.rem))
+    _lib.check(rc, entry)
+
+
+def rms_norm(x: Tensor, gamma: Tensor, eps: float) -> Tensor:
+    """``bf16(x * rsqrt(mean(x^2) + eps) * gamma)`` over the last dimension, one rounding: the
+    arithmetic (reduction order included) of the RMSNorm that :func:`gemv_bf16_grouped` fuses."""
+    lib = _lib.load()
+    K = x.shape[-1]
+    flat = x.reshape(-1, K).contiguous()
+    out = torch.empty_like(flat)
+    g = _req(gamma.contiguous(), torch.bfloat16, "gamma", flat)
+    with torch.cuda.device(flat.device):
+        for r0 in range(0, flat.shape[0], X_TRANSFORM_MAX_ROWS):
+            rows = flat[r0:r0 + X_TRANSFORM_MAX_ROWS]
+            _lib.check(lib.bhi_rms_norm(_req(rows, torch.bfloat16, "x"), g, out[r0:].data_ptr(), rows.shape[0], K, float(eps),
+                                        _stream(flat)), "rms_norm")
+    return out.view(x.shape)
+
+
+def silu_mul(gate: Tensor, up: Tensor) -> Tensor:
+    """``bf16(bf16(silu(gate)) * up)``: the roundings of a BF16 ``F.silu(gate) * up``, as the GEMV
+    fuses them."""
+    if gate.shape != up.shape:
+        raise RuntimeError("gate and up must have one shape")
+    g, u = gate.contiguous(), up.contiguous()
+    out = torch.empty_like(g)
+    with torch.cuda.device(g.device):
+        _lib.check(_lib.load().bhi_silu_mul(_req(g, torch.bfloat16, "gate"), _req(u, torch.bfloat16, "up", g), out.data_ptr(),
+                                            g.numel(), _stream(g)), "silu_mul")
+    return out
 
 
 def _fill_member(m, w, Y: Tensor, bias, ref: Tensor) -> bool:

@@ -150,13 +150,34 @@ typedef struct bhi_gemv_member {
     const void* bias;
     int32_t M;
     int32_t reserved;
-} bhi_gemv_member;                 /* 80 bytes: nine 8-byte fields, two ints */
+    const void* residual;          /* bf16 [batch, M] or NULL: added after the bias, as a separate BF16
+                                    * `y + residual` (the residual connection around the layer) would */
+} bhi_gemv_member;                 /* 88 bytes: nine 8-byte fields, two ints, one 8-byte field */
 int bhi_gemv_bf16_huffman_grouped(const bhi_gemv_member* members, int n_members, const void* X,
                                   int split_k, int Ks, int batch, void* stream);
 int bhi_gemv_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, const void* X,
                               int split_k, int Ks, int batch, void* stream);
 int bhi_gemv_bf16_nibble_grouped(const bhi_gemv_member* members, int n_members, const void* X,
                                  int split_k, int Ks, int batch, void* stream);
+
+/* Grouped GEMV on a FUNCTION of X, so that the layer in front of the linear needs no kernel
+ * (and no round trip through memory) of its own -- the reference runs these as separate
+ * PyTorch kernels around its op (functional.py:403-404 is the only fusion point it has):
+ *   x_mode 1  RMSNorm:  h = x * rsqrt(mean(x^2) + eps) * gamma,  x_aux = gamma bf16 [split_k*Ks]
+ *   x_mode 2  SwiGLU:   h = silu(gate) * x,                      x_aux = gate  bf16 [batch, split_k*Ks]
+ *   x_mode 0  h = x (the plain grouped entry points)
+ * batch <= 4.  The roundings are those of bhi_rms_norm / bhi_silu_mul below followed by the
+ * plain GEMV: the fused and the unfused sequence give the same bits. */
+int bhi_gemv_bf16_huffman_grouped_x(const bhi_gemv_member* members, int n_members, const void* X,
+                                    int split_k, int Ks, int batch, int x_mode, const void* x_aux, float eps,
+                                    void* stream);
+int bhi_gemv_bf16_ans_grouped_x(const bhi_gemv_member* members, int n_members, const void* X,
+                                int split_k, int Ks, int batch, int x_mode, const void* x_aux, float eps,
+                                void* stream);
+/* The same two pieces as kernels of their own (1..4 rows; out may not alias the inputs of
+ * bhi_rms_norm): out = bf16(x * r * gamma) with one rounding; out = bf16(bf16(silu(gate)) * up). */
+int bhi_rms_norm(const void* X, const void* gamma, void* out, int rows, int K, float eps, void* stream);
+int bhi_silu_mul(const void* gate, const void* up, void* out, int64_t n, void* stream);
 
 /* Fused decode + matrix product for 1..32 rows of X (meant for 9..32; up to 8 the GEMV
  * entry points are faster): Y = X W^T (+ bias) with the weights going from the decoder's
