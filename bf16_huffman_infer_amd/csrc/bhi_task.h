@@ -180,15 +180,48 @@ __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
 // `acc` within three wait states of the write, and the compiler, which does not see a dot
 // product here, will happily copy `acc` to another register right behind the statement
 // (wrong sums, in whichever batch row the copy happened to hit).  Hence the closing s_nop.
-__device__ __forceinline__ void dot_quad4(float& acc, uint32_t x, const uint32_t (&w)[4]) {
-    asm("s_nop 1\n\t"
-        "v_dot2c_f32_bf16_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf\n\t"
-        "v_dot2c_f32_bf16_dpp %0, %1, %3 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
-        "v_dot2c_f32_bf16_dpp %0, %1, %4 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
-        "v_dot2c_f32_bf16_dpp %0, %1, %5 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 2"
-        : "+v"(acc) : "v"(x), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+#define BHI_DOT(ACC, X, W, Q) "v_dot2c_f32_bf16_dpp " ACC ", " X ", " W " quad_perm:[" Q "," Q "," Q "," Q "] row_mask:0xf bank_mask:0xf\n\t"
+// N batch rows at once (N <= 4): acc[j] += the four products of x[j] with w[0..3].  One
+// statement for all of them, so that the two s_nops are paid once per step and not once per
+// batch row, and the products of different rows interleave (no instruction waits for the one
+// right before it).
+template <int N>
+__device__ __forceinline__ void dot_rows(float* acc, const uint32_t (&x)[4], const uint32_t (&w)[4]) {
+    static_assert(N >= 1 && N <= 4, "up to four batch rows per statement");
+    if constexpr (N == 1) {
+        asm("s_nop 1\n\t"
+            BHI_DOT("%0", "%1", "%2", "0") BHI_DOT("%0", "%1", "%3", "1") BHI_DOT("%0", "%1", "%4", "2") BHI_DOT("%0", "%1", "%5", "3")
+            "s_nop 2"
+            : "+v"(acc[0]) : "v"(x[0]), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+    } else if constexpr (N == 2) {
+        asm("s_nop 1\n\t"
+            BHI_DOT("%0", "%2", "%4", "0") BHI_DOT("%1", "%3", "%4", "0")
+            BHI_DOT("%0", "%2", "%5", "1") BHI_DOT("%1", "%3", "%5", "1")
+            BHI_DOT("%0", "%2", "%6", "2") BHI_DOT("%1", "%3", "%6", "2")
+            BHI_DOT("%0", "%2", "%7", "3") BHI_DOT("%1", "%3", "%7", "3")
+            "s_nop 2"
+            : "+v"(acc[0]), "+v"(acc[1]) : "v"(x[0]), "v"(x[1]), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+    } else if constexpr (N == 3) {
+        asm("s_nop 1\n\t"
+            BHI_DOT("%0", "%3", "%6", "0") BHI_DOT("%1", "%4", "%6", "0") BHI_DOT("%2", "%5", "%6", "0")
+            BHI_DOT("%0", "%3", "%7", "1") BHI_DOT("%1", "%4", "%7", "1") BHI_DOT("%2", "%5", "%7", "1")
+            BHI_DOT("%0", "%3", "%8", "2") BHI_DOT("%1", "%4", "%8", "2") BHI_DOT("%2", "%5", "%8", "2")
+            BHI_DOT("%0", "%3", "%9", "3") BHI_DOT("%1", "%4", "%9", "3") BHI_DOT("%2", "%5", "%9", "3")
+            "s_nop 2"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2])
+            : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+    } else {
+        asm("s_nop 1\n\t"
+            BHI_DOT("%0", "%4", "%8", "0") BHI_DOT("%1", "%5", "%8", "0") BHI_DOT("%2", "%6", "%8", "0") BHI_DOT("%3", "%7", "%8", "0")
+            BHI_DOT("%0", "%4", "%9", "1") BHI_DOT("%1", "%5", "%9", "1") BHI_DOT("%2", "%6", "%9", "1") BHI_DOT("%3", "%7", "%9", "1")
+            BHI_DOT("%0", "%4", "%10", "2") BHI_DOT("%1", "%5", "%10", "2") BHI_DOT("%2", "%6", "%10", "2") BHI_DOT("%3", "%7", "%10", "2")
+            BHI_DOT("%0", "%4", "%11", "3") BHI_DOT("%1", "%5", "%11", "3") BHI_DOT("%2", "%6", "%11", "3") BHI_DOT("%3", "%7", "%11", "3")
+            "s_nop 2"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])
+            : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+    }
 }
+#undef BHI_DOT
 
 // What the GEMV multiplies the weights with: X as given, or a function of X that the layer in
 // front of the linear would otherwise have to write to memory with a kernel of its own:
@@ -342,10 +375,8 @@ struct DotPolicy {
 #pragma unroll
                 for (int j = 0; j < BS && j < 4; ++j) xb[j] = silu_mul_pair(gb[j], xb[j]);
             }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (4 * q + j < BS) dot_quad4(dot[4 * q + j], xb[j], w);
-            }
+            if (q == 0) dot_rows<(BS < 4 ? BS : 4)>(dot, xb, w);
+            else dot_rows<(BS > 4 ? BS - 4 : 1)>(dot + 4, xb, w);
         }
         if (PIPED) xload(xr[s.i % XAHEAD], s.t + XAHEAD);
     }
