@@ -1,4 +1,5 @@
-"""The six custom ops of namespace ``bf16_huffman_infer`` on HIP (plus three for the nibble codec).
+"""The six custom ops of namespace ``bf16_huffman_infer`` on HIP (the nibble codec's three live in a
+namespace of their own, ``bf16_huffman_infer_amd``: the reference's namespace carries the reference's schemas only).
 
 Same op names, schemas and positional wrappers as the reference
 (``bf16_huffman_infer/src/bf16_huffman_infer.cpp:29-35``, ``ops.py:6-61``).  The schemas
@@ -24,10 +25,11 @@ _LIB.define("huffman_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor off
 _LIB.define("gemv_bf16_ans(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
 _LIB.define("ans_encode(Tensor data, Tensor freq, Tensor cum, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
 _LIB.define("ans_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
-# not in the reference: the fixed-width codec, with the rANS ops' shapes
-_LIB.define("gemv_bf16_nibble(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
-_LIB.define("nibble_encode(Tensor data, Tensor LUT, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
-_LIB.define("nibble_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
+# not in the reference, hence not in its namespace: the fixed-width codec, with the rANS ops' shapes
+_EXTRA = torch.library.Library("bf16_huffman_infer_amd", "DEF")
+_EXTRA.define("gemv_bf16_nibble(Tensor A_rem, Tensor A_exp, Tensor X, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
+_EXTRA.define("nibble_encode(Tensor data, Tensor LUT, Tensor(a!) output, Tensor(b!) output_lengths) -> ()")
+_EXTRA.define("nibble_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor offsets, Tensor LUT) -> ()")
 
 LANE_BYTES_PER_STEP = 512          # 64 lanes x 8 exponent bytes
 
@@ -204,7 +206,7 @@ def _nibble_encode(data, LUT, output, output_lengths):
 
 for _name, _fn in (("gemv_bf16_nibble", _gemv_bf16_nibble), ("nibble_encode", _nibble_encode),
                    ("nibble_decode", _nibble_decode)):
-    _LIB.impl(_name, _fn, "CUDA")
+    _EXTRA.impl(_name, _fn, "CUDA")
 
 for _name, _fn in (("gemv_bf16_huffman", _gemv_bf16_huffman), ("huffman_encode", _huffman_encode),
                    ("huffman_decode", _huffman_decode), ("gemv_bf16_ans", _gemv_bf16_ans),
@@ -258,15 +260,15 @@ def ans_encode_capacity(n_steps: int) -> int:
 
 
 def gemv_bf16_nibble(A_rem: Tensor, A_exp: Tensor, X: Tensor, Y: Tensor, offsets: Tensor, LUT: Tensor) -> None:
-    torch.ops.bf16_huffman_infer.gemv_bf16_nibble.default(A_rem, A_exp, X, Y, offsets, LUT)
+    torch.ops.bf16_huffman_infer_amd.gemv_bf16_nibble.default(A_rem, A_exp, X, Y, offsets, LUT)
 
 
 def nibble_encode(data: Tensor, LUT: Tensor, output: Tensor, output_lengths: Tensor) -> None:
-    torch.ops.bf16_huffman_infer.nibble_encode.default(data, LUT, output, output_lengths)
+    torch.ops.bf16_huffman_infer_amd.nibble_encode.default(data, LUT, output, output_lengths)
 
 
 def nibble_decode(A_rem: Tensor, A_exp: Tensor, Y: Tensor, offsets: Tensor, LUT: Tensor) -> None:
-    torch.ops.bf16_huffman_infer.nibble_decode.default(A_rem, A_exp, Y, offsets, LUT)
+    torch.ops.bf16_huffman_infer_amd.nibble_decode.default(A_rem, A_exp, Y, offsets, LUT)
 
 
 X_PLAIN, X_RMS, X_SILU_MUL = 0, 1, 2
