@@ -20,6 +20,8 @@ struct AnsCodec {
     static constexpr bool kPersistent = true;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = kAnsTableWords;
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__) { return false; }
+    static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__) { return 0u; }
+    static __device__ __forceinline__ bool variant_test(uint32_t, const uint8_t* __restrict__) { return false; }
 };
 
 // What the encoder does to a state for one half-step, backwards over its four symbols.

@@ -71,6 +71,27 @@ __device__ __forceinline__ uint32_t rebuild_pair(uint32_t e, uint32_t z) {
 __device__ __forceinline__ uint32_t rem_lo_pair(uint32_t r) { return __builtin_amdgcn_perm(r, r, 0x01010000u); }
 __device__ __forceinline__ uint32_t rem_hi_pair(uint32_t r) { return __builtin_amdgcn_perm(r, r, 0x03030202u); }
 
+// A word of memory that nothing writes while the kernel runs (offsets, the format header),
+// read at a wave-uniform address: through the constant address space the compiler issues a
+// scalar load, which neither queues behind the vector loads in flight nor has to be waited
+// for with them.  At a lane-dependent address it is an ordinary vector load.
+typedef __attribute__((address_space(4))) const uint32_t const_u32;
+__device__ __forceinline__ uint32_t constant_word(const uint32_t* p) {
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wold-style-cast"
+    return *(const_u32*)p;
+#pragma clang diagnostic pop
+}
+
+// A block barrier that orders LDS traffic only.  __syncthreads() also waits for every global
+// load in flight (s_waitcnt vmcnt(0)), which would drain the prefetched windows at each barrier.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): this wavefront's LDS writes have landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // Position of a task's stream and of the stream that follows it in (k, g, c) order.
 struct TaskSpan { uint32_t base, end; };
 
@@ -78,10 +99,10 @@ __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offse
                                               int k, int g, int c, uint32_t total_words) {
     TaskSpan s;
     const int G = M / kGroupRows;
-    s.base = offsets[(size_t)k * M + kGroupRows * g + c];
-    if (c + 1 < nc)            s.end = offsets[(size_t)k * M + kGroupRows * g + c + 1];
-    else if (g + 1 < G)        s.end = offsets[(size_t)k * M + kGroupRows * (g + 1)];
-    else if (k + 1 < split_k)  s.end = offsets[(size_t)(k + 1) * M];
+    s.base = constant_word(offsets + (size_t)k * M + kGroupRows * g + c);
+    if (c + 1 < nc)            s.end = constant_word(offsets + (size_t)k * M + kGroupRows * g + c + 1);
+    else if (g + 1 < G)        s.end = constant_word(offsets + (size_t)k * M + kGroupRows * (g + 1));
+    else if (k + 1 < split_k)  s.end = constant_word(offsets + (size_t)(k + 1) * M);
     else                       s.end = total_words;
     return s;
 }

@@ -17,6 +17,8 @@ struct HuffCodec {
     static constexpr int kTableWords = kTableEntries;
     // escaped pairs need the slower walk; the header says whether the matrix has any
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ header) { return header_has_esc(header); }
+    static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__ header) { return header_flag_word(header); }
+    static __device__ __forceinline__ bool variant_test(uint32_t w, const uint8_t* __restrict__ header) { return header_flag_test(w, header); }
 };
 
 // ------------------------------------------------------------------ encoder

@@ -49,15 +49,6 @@ constexpr int kMmaMaxBatch = 32;
 constexpr int kMmaMaxSlices = 8;
 constexpr int kMmaSliceBelowGroups = 2048;   // weights with fewer row groups are cut along K
 
-// A block barrier that orders LDS traffic only.  __syncthreads() also waits for every global
-// load in flight (s_waitcnt vmcnt(0)), which would drain the prefetched windows at each barrier.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0): this wavefront's LDS writes have landed
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
 template <int Q>
 struct MmaPolicy {
     struct Slot { uint2 rem; };

@@ -17,9 +17,11 @@ struct NibbleCodec {
     static constexpr bool kTransformsX = false;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr bool kPersistent = false;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = 4;          // base and flags, one 16-byte copy
-    static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ lut) {
-        return uniform(((const uint32_t*)lut)[1]) != 0;
+    static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__ lut) {
+        return constant_word((const uint32_t*)lut + 1);
     }
+    static __device__ __forceinline__ bool variant_test(uint32_t w, const uint8_t* __restrict__) { return w != 0; }
+    static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ lut) { return variant_test(variant_word(lut), lut); }
 };
 
 // One wavefront per task: pass 1 counts escapes, pass 2 writes the rows and the escape

@@ -20,9 +20,32 @@ __device__ __forceinline__ void load_table(uint32_t* __restrict__ lds, const uin
     for (int i = threadIdx.x; i < WORDS / 4; i += blockDim.x) dst[i] = src[i];
 }
 
+// The same copy in two halves: the loads are issued when a block starts, ahead of every
+// other load (vector loads return in issue order, so the table arrives first), and the LDS
+// writes follow once the task's own first loads are on their way.
+template <int WORDS, int THREADS>
+struct TableCopy {
+    static constexpr int kVecs = WORDS / 4;
+    static_assert(kVecs <= 2 * THREADS, "at most two 16-byte pieces per thread");
+    // named registers: an array that a lambda captures by reference ends up in scratch memory
+    typedef uint32_t vec_t __attribute__((ext_vector_type(4)));
+    vec_t v0, v1;
+    __device__ __forceinline__ void issue(const uint32_t* __restrict__ g) {
+        const int i = (int)threadIdx.x;
+        if (kVecs >= THREADS || i < kVecs) v0 = ((const vec_t*)g)[i];
+        if (kVecs > THREADS && (kVecs == 2 * THREADS || i + THREADS < kVecs)) v1 = ((const vec_t*)g)[i + THREADS];
+    }
+    __device__ __forceinline__ void commit(uint32_t* __restrict__ lds) const {
+        const int i = (int)threadIdx.x;
+        if (kVecs >= THREADS || i < kVecs) ((vec_t*)lds)[i] = v0;
+        if (kVecs > THREADS && (kVecs == 2 * THREADS || i + THREADS < kVecs)) ((vec_t*)lds)[i + THREADS] = v1;
+    }
+};
+
 struct Shape {
     int M, Ks, split_k, nc, steps;      // steps per (split, group)
     uint32_t total_words;
+    int nc_log2;                        // nc is a power of two (chunks_per_group doubles it)
 };
 
 // One segment of a task: S steps whose operands a policy has loaded into `slot`.
@@ -65,24 +88,28 @@ __device__ __forceinline__ void run_segment(Cursor& cur, const uint32_t* lut, Po
     decode_segment<true, HAS_ESC>(cur, lut, pol, now, seg, ns);
 }
 
-// The walk over one task.  Its first loads (operands of the first segment, the rows that
-// prime the ring) are issued before `between()` runs, which is where the first task of a
-// block copies the decode table into LDS: table, rows and operands are in flight
-// together.  Whole segments alternate between two operand sets (one being decoded, one in
-// flight); the last whole segment reloads itself instead of running past the task.  A
-// last, shorter segment clamps its step indices and guards its steps.
-template <bool HAS_ESC, int S, class Cursor, class Policy, class Between>
-__device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between) {
-    typename Policy::Slot a[S], b[S];
-    const int full_end = ns - ns % S;
-    const int last_full = full_end - S;
+// The walk over one task, in two halves.  `open_task` issues the task's first loads (operands
+// of the first segment, the rows that prime the ring) and then runs `between()`, which is
+// where the first task of a block copies the decode table into LDS: table, rows and operands
+// are in flight together.  It does not depend on the codec's variant, so a caller can issue it
+// before the flag that selects the variant has arrived.  `walk_task` then alternates whole
+// segments between two operand sets (one being decoded, one in flight); the last whole segment
+// reloads itself instead of running past the task.  A last, shorter segment clamps its step
+// indices and guards its steps.
+template <int S, class Policy>
+struct TaskOpen {
+    typename Policy::Slot a[S];
+    uint32_t rows[S];
+    bool pending;
+};
+
+template <int S, class Cursor, class Policy, class Between>
+__device__ __forceinline__ void open_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between,
+                                          TaskOpen<S, Policy>& o) {
     pol.prime();
-    if (full_end > 0) {
-        pol.load_full(a, 0);
-    } else {
+    // clamped step indices: a task shorter than a segment loads its last step again
 #pragma unroll
-        for (int i = 0; i < S; ++i) pol.load(a[i], i);
-    }
+    for (int i = 0; i < S; ++i) pol.load(o.a[i], i);
     {
         uint32_t first[kPrimeRows];
         cur.prime_issue(first);
@@ -90,34 +117,63 @@ __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Polic
         cur.prime_commit(first);
     }
     cur.start(lut);
-    uint32_t rows[S];
-    bool pending = cur.template room<S>();
-    if (pending) cur.prefetch(rows);
+    o.pending = cur.template room<S>();
+    if (o.pending) cur.prefetch(o.rows);
+}
+
+template <bool HAS_ESC, int S, class Cursor, class Policy>
+__device__ __forceinline__ void walk_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, TaskOpen<S, Policy>& o) {
+    typename Policy::Slot b[S];
+    const int full_end = ns - ns % S;
+    const int last_full = full_end - S;
     int seg = 0;
     if (full_end > 0) {
         for (;;) {
             int nx = seg + S;
-            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, ns);
+            run_segment<HAS_ESC, S>(cur, lut, pol, o.pending, o.rows, o.a, b, seg, nx < last_full ? nx : last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
             nx = seg + S;
-            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, ns);
+            run_segment<HAS_ESC, S>(cur, lut, pol, o.pending, o.rows, b, o.a, seg, nx < last_full ? nx : last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
         }
         if (seg < ns) {
 #pragma unroll
-            for (int i = 0; i < S; ++i) pol.load(a[i], seg + i);
+            for (int i = 0; i < S; ++i) pol.load(o.a[i], seg + i);
         }
     }
-    if (pending) cur.commit(rows);
-    if (seg < ns) decode_segment<false, HAS_ESC, S>(cur, lut, pol, a, seg, ns);
+    if (o.pending) cur.commit(o.rows);
+    if (seg < ns) decode_segment<false, HAS_ESC, S>(cur, lut, pol, o.a, seg, ns);
+}
+
+template <bool HAS_ESC, int S, class Cursor, class Policy, class Between>
+__device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between) {
+    TaskOpen<S, Policy> o;
+    open_task<S>(cur, lut, pol, ns, between, o);
+    walk_task<HAS_ESC, S>(cur, lut, pol, ns, o);
 }
 
 // The format header (code_lengths buffer): [0] version, [1] table bits, [2] ESC code
 // length, [3] nonzero when the matrix contains escaped pairs.
+// The flag is read in two halves so that a kernel can issue the load early and look at the
+// word late: `flag_word` is the aligned word that holds byte 3 (a scalar load needs a word
+// address), `flag_test` picks the byte out of it.
+__device__ __forceinline__ uint32_t header_flag_word(const uint8_t* __restrict__ header) {
+    return constant_word((const uint32_t*)((uintptr_t)(header + 3) & ~(uintptr_t)3));
+}
+__device__ __forceinline__ bool header_flag_test(uint32_t w, const uint8_t* __restrict__ header) {
+    return ((w >> (8u * (uint32_t)((uintptr_t)(header + 3) & 3))) & 0xFFu) != 0;
+}
 __device__ __forceinline__ bool header_has_esc(const uint8_t* __restrict__ header) {
-    return uniform(header[3]) != 0;
+    return header_flag_test(header_flag_word(header), header);
+}
+
+// Pins a wave-uniform value where it stands: what is computed from it cannot move above this
+// point, so the wait for the load behind it lands here and not right after the load.
+__device__ __forceinline__ uint32_t pin_uniform(uint32_t v) {
+    asm volatile("" : "+s"(v));
+    return v;
 }
 
 // decode-to-BF16: rem in, 16 bytes of weights out per lane and step
@@ -405,10 +461,11 @@ struct TaskId { int k, c, t0, t1; };
 
 __device__ __forceinline__ TaskId task_of(const Shape& s, int kc) {
     TaskId id;
-    id.k = kc / s.nc;
-    id.c = kc % s.nc;
-    id.t0 = (s.steps * id.c) / s.nc;
-    id.t1 = (s.steps * (id.c + 1)) / s.nc;
+    // shifts, not divisions: every wavefront runs this before its first load
+    id.k = kc >> s.nc_log2;
+    id.c = kc & (s.nc - 1);
+    id.t0 = (s.steps * id.c) >> s.nc_log2;
+    id.t1 = (s.steps * (id.c + 1)) >> s.nc_log2;
     return id;
 }
 
@@ -518,15 +575,22 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     const int block = (int)blockIdx.x - mb.first_block;
     // P wavefronts share one row group; a block holds NW / P row groups
     const int P = s.split_k * s.nc < NW ? s.split_k * s.nc : NW;
-    const int groups_per_block = NW / P;
+    static_assert(NW == 4, "the wavefront-to-task arithmetic below is written for four wavefronts");
+    const int groups_per_block = P == 1 ? 4 : (P == 2 ? 2 : 1);
     // The table reaches LDS while the first task's first loads are in flight: the copy and
     // its barrier run once per wavefront, inside the first task or, for a wavefront
     // without one, right after.
     bool staged = false;
+    // (the RMSNorm variant needs its registers for the sums of squares at that point and
+    // copies the table in one go instead)
+    constexpr bool kEarlyTable = XM != kXRms;
+    TableCopy<Codec::kTableWords, NW * kLanes> table_copy;
+    if (kEarlyTable) table_copy.issue(table);
     auto stage_table = [&]() {
         if (!staged) {
-            load_table<Codec::kTableWords>(lut, table);
-            __syncthreads();
+            if (kEarlyTable) table_copy.commit(lut);
+            else load_table<Codec::kTableWords>(lut, table);
+            lds_barrier();
             staged = true;
         }
     };
@@ -535,11 +599,13 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
     const int wave = (int)uniform(threadIdx.x / kLanes);
     const int G = s.M / kGroupRows;
     const int per_group = s.split_k * s.nc;
-    const int rg = wave / P, p = wave % P;
+    // wave / P and wave % P for wave < 4 and P in 1..4 without a division
+    const int rg = P == 1 ? wave : (P == 2 ? wave >> 1 : (wave >= P ? 1 : 0));
+    const int p = wave - rg * P;
     const int g = block * groups_per_block + rg;
     const bool active = rg < groups_per_block && g < G;
     const int K = s.Ks * s.split_k;
-    const bool variant = Codec::variant(header);
+    const uint32_t variant_word = Codec::variant_word(header);
 
     DotPolicy<BS, XM> pol;
     constexpr int NSET = DotPolicy<BS, XM>::NSET;
@@ -569,8 +635,18 @@ void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
             pol.aq0 = XM == kXPlain ? nullptr
                                     : (const uint32_t*)(grp.xaux + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
-            if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
-            else run_task<false, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
+            // the first loads go out before the variant flag is looked at: its load is in
+            // flight with the offsets', and nothing waits for it until the walk begins
+            TaskOpen<S, DotPolicy<BS, XM>> o;
+            open_task<S>(cur, lut, pol, id.t1 - id.t0, stage_all, o);
+            const bool variant = Codec::variant_test(pin_uniform(variant_word), header);
+            if (variant) walk_task<true, S>(cur, lut, pol, id.t1 - id.t0, o);
+            else walk_task<false, S>(cur, lut, pol, id.t1 - id.t0, o);
+            // Nothing is in flight at the end of a task.  Saying so keeps the compiler from
+            // waiting at the top of the loop for loads that a previous pass might have left
+            // behind: on the first pass that wait would be for the table, before the task's
+            // own first loads are issued.
+            __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         pol.fold();
         // lane 4*b + j holds, in register i, the sum of row i for batch j over column block b
@@ -643,6 +719,9 @@ static inline int check_shape(int split_k, int M, int Ks, int64_t exp_words, bhi
     s->M = M; s->Ks = Ks; s->split_k = split_k;
     s->nc = chunks_per_group(M, Ks, split_k);
     s->steps = Ks / kStepCols;
+    s->nc_log2 = 0;
+    while ((1 << s->nc_log2) < s->nc) ++s->nc_log2;
+    if ((1 << s->nc_log2) != s->nc) return bhi_fail(BHI_ELAYOUT, "chunks per group must be a power of two");
     if ((s->steps + s->nc - 1) / s->nc > kMaxTaskSteps)
         return bhi_fail(BHI_ELAYOUT, "more than 128 steps per task");
     s->total_words = (uint32_t)(exp_words - kTailPadWords);
