@@ -553,15 +553,20 @@ __device__ __forceinline__ uint16_t finish_output(float sum, const uint16_t* __r
 
 template <class Codec, int BS, int NW, int S, int XM = kXPlain>
 __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
-void gemv_kernel(const uint16_t* __restrict__ X, const Group grp) {
+void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int first3, const Group grp) {
     // The partial sums reuse the rings once every task of the block is done.
     __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
     __shared__ float rms_part[XM == kXRms ? NW * BS : 1];
+    // first1..3: first block of members 1..3 (INT_MAX when absent).  Leading scalar arguments
+    // are in registers when the wavefront starts (the library is built with kernel-argument
+    // preload), so the member is known without a fetch and its fields take one fetch, not two
+    // dependent ones.
+    static_assert(kMaxMembers == 4, "one leading argument per member after the first");
     int member = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxMembers; ++i)
-        if (i < grp.n && (int)blockIdx.x >= grp.m[i].first_block) member = i;
+    if ((int)blockIdx.x >= first1) member = 1;
+    if ((int)blockIdx.x >= first2) member = 2;
+    if ((int)blockIdx.x >= first3) member = 3;
     const Member& mb = grp.m[member];
     const uint8_t* __restrict__ A_rem = mb.rem;
     const uint32_t* __restrict__ A_exp = mb.exp;
@@ -741,6 +746,8 @@ static inline int gemv_blocks(const bhi::Shape& s) {
 // of 8 or 16 steps in any case.  A launch with more wavefronts than the GPU holds (a group
 // of weights) runs at full contention for most of its time; there, on long tasks (28
 // steps), the smaller per-step overhead of long segments wins by about 5 %.
+static inline int first_block_of(const bhi::Group& g, int i) { return i < g.n ? g.m[i].first_block : 0x7FFFFFFF; }
+
 constexpr int kLongTaskSteps = 24;
 template <class Codec, int BS>
 static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks, hipStream_t stream) {
@@ -748,9 +755,9 @@ static inline void launch_gemv(const void* X, const bhi::Group& grp, int blocks,
     const dim3 grid((unsigned)blocks), block(kWavesPerBlock * kLanes);
     const Shape& s0 = grp.m[0].s;
     if ((long long)blocks * kWavesPerBlock > kTargetTasks && s0.steps / s0.nc >= kLongTaskSteps)
-        hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegLong>), grid, block, 0, stream, (const uint16_t*)X, grp);
+        hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegLong>), grid, block, 0, stream, (const uint16_t*)X, first_block_of(grp, 1), first_block_of(grp, 2), first_block_of(grp, 3), grp);
     else
-        hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegShort>), grid, block, 0, stream, (const uint16_t*)X, grp);
+        hipLaunchKernelGGL((bhi::gemv_kernel<Codec, BS, kWavesPerBlock, kSegShort>), grid, block, 0, stream, (const uint16_t*)X, first_block_of(grp, 1), first_block_of(grp, 2), first_block_of(grp, 3), grp);
 }
 
 // Launches with a transformed X (kXRms, kXSiluMul): batch 1..4, short segments.
@@ -760,10 +767,10 @@ static inline void launch_gemv_x(int batch, const void* X, const bhi::Group& grp
     const dim3 grid((unsigned)blocks), block(kWavesPerBlock * kLanes);
     const uint16_t* x = (const uint16_t*)X;
     switch (batch) {
-        case 1: hipLaunchKernelGGL((gemv_kernel<Codec, 1, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
-        case 2: hipLaunchKernelGGL((gemv_kernel<Codec, 2, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
-        case 3: hipLaunchKernelGGL((gemv_kernel<Codec, 3, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
-        default: hipLaunchKernelGGL((gemv_kernel<Codec, 4, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, grp); break;
+        case 1: hipLaunchKernelGGL((gemv_kernel<Codec, 1, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, first_block_of(grp, 1), first_block_of(grp, 2), first_block_of(grp, 3), grp); break;
+        case 2: hipLaunchKernelGGL((gemv_kernel<Codec, 2, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, first_block_of(grp, 1), first_block_of(grp, 2), first_block_of(grp, 3), grp); break;
+        case 3: hipLaunchKernelGGL((gemv_kernel<Codec, 3, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, first_block_of(grp, 1), first_block_of(grp, 2), first_block_of(grp, 3), grp); break;
+        default: hipLaunchKernelGGL((gemv_kernel<Codec, 4, kWavesPerBlock, kSegShort, XM>), grid, block, 0, stream, x, first_block_of(grp, 1), first_block_of(grp, 2), first_block_of(grp, 3), grp); break;
     }
 }
 

@@ -10,6 +10,9 @@ LIB = os.path.join(PKG, "libbhi_hip.so")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first five dwords of every kernel's arguments arrive in registers (the fused GEMV
+    # picks its group member from them before its first memory access)
+    "-mllvm", "-amdgpu-kernarg-preload-count=5",
     "-Wall", "-Wno-unused-variable",
 ]
 
