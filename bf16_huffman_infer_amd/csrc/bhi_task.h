@@ -88,28 +88,24 @@ __device__ __forceinline__ void run_segment(Cursor& cur, const uint32_t* lut, Po
     decode_segment<true, HAS_ESC>(cur, lut, pol, now, seg, ns);
 }
 
-// The walk over one task, in two halves.  `open_task` issues the task's first loads (operands
-// of the first segment, the rows that prime the ring) and then runs `between()`, which is
-// where the first task of a block copies the decode table into LDS: table, rows and operands
-// are in flight together.  It does not depend on the codec's variant, so a caller can issue it
-// before the flag that selects the variant has arrived.  `walk_task` then alternates whole
-// segments between two operand sets (one being decoded, one in flight); the last whole segment
-// reloads itself instead of running past the task.  A last, shorter segment clamps its step
-// indices and guards its steps.
-template <int S, class Policy>
-struct TaskOpen {
-    typename Policy::Slot a[S];
-    uint32_t rows[S];
-    bool pending;
-};
-
-template <int S, class Cursor, class Policy, class Between>
-__device__ __forceinline__ void open_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between,
-                                          TaskOpen<S, Policy>& o) {
+// The walk over one task.  Its first loads (operands of the first segment, the rows that
+// prime the ring) are issued before `between()` runs, which is where the first task of a
+// block stores the decode table into LDS: table, rows and operands are in flight
+// together.  Whole segments alternate between two operand sets (one being decoded, one in
+// flight); the last whole segment reloads itself instead of running past the task.  A
+// last, shorter segment clamps its step indices and guards its steps.
+template <bool HAS_ESC, int S, class Cursor, class Policy, class Between>
+__device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between) {
+    typename Policy::Slot a[S], b[S];
+    const int full_end = ns - ns % S;
+    const int last_full = full_end - S;
     pol.prime();
-    // clamped step indices: a task shorter than a segment loads its last step again
+    if (full_end > 0) {
+        pol.load_full(a, 0);
+    } else {
 #pragma unroll
-    for (int i = 0; i < S; ++i) pol.load(o.a[i], i);
+        for (int i = 0; i < S; ++i) pol.load(a[i], i);
+    }
     {
         uint32_t first[kPrimeRows];
         cur.prime_issue(first);
@@ -117,48 +113,35 @@ __device__ __forceinline__ void open_task(Cursor& cur, const uint32_t* lut, Poli
         cur.prime_commit(first);
     }
     cur.start(lut);
-    o.pending = cur.template room<S>();
-    if (o.pending) cur.prefetch(o.rows);
-}
-
-template <bool HAS_ESC, int S, class Cursor, class Policy>
-__device__ __forceinline__ void walk_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, TaskOpen<S, Policy>& o) {
-    typename Policy::Slot b[S];
-    const int full_end = ns - ns % S;
-    const int last_full = full_end - S;
+    uint32_t rows[S];
+    bool pending = cur.template room<S>();
+    if (pending) cur.prefetch(rows);
     int seg = 0;
     if (full_end > 0) {
         for (;;) {
             int nx = seg + S;
-            run_segment<HAS_ESC, S>(cur, lut, pol, o.pending, o.rows, o.a, b, seg, nx < last_full ? nx : last_full, ns);
+            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
             nx = seg + S;
-            run_segment<HAS_ESC, S>(cur, lut, pol, o.pending, o.rows, b, o.a, seg, nx < last_full ? nx : last_full, ns);
+            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
         }
         if (seg < ns) {
 #pragma unroll
-            for (int i = 0; i < S; ++i) pol.load(o.a[i], seg + i);
+            for (int i = 0; i < S; ++i) pol.load(a[i], seg + i);
         }
     }
-    if (o.pending) cur.commit(o.rows);
-    if (seg < ns) decode_segment<false, HAS_ESC, S>(cur, lut, pol, o.a, seg, ns);
-}
-
-template <bool HAS_ESC, int S, class Cursor, class Policy, class Between>
-__device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Policy& pol, int ns, Between between) {
-    TaskOpen<S, Policy> o;
-    open_task<S>(cur, lut, pol, ns, between, o);
-    walk_task<HAS_ESC, S>(cur, lut, pol, ns, o);
+    if (pending) cur.commit(rows);
+    if (seg < ns) decode_segment<false, HAS_ESC, S>(cur, lut, pol, a, seg, ns);
 }
 
 // The format header (code_lengths buffer): [0] version, [1] table bits, [2] ESC code
 // length, [3] nonzero when the matrix contains escaped pairs.
 // The flag is read in two halves so that a kernel can issue the load early and look at the
-// word late: `flag_word` is the aligned word that holds byte 3 (a scalar load needs a word
-// address), `flag_test` picks the byte out of it.
+// word late: `header_flag_word` is the aligned word that holds byte 3 (a scalar load needs a
+// word address), `header_flag_test` picks the byte out of it.
 __device__ __forceinline__ uint32_t header_flag_word(const uint8_t* __restrict__ header) {
     return constant_word((const uint32_t*)((uintptr_t)(header + 3) & ~(uintptr_t)3));
 }
@@ -640,13 +623,10 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
             pol.aq0 = XM == kXPlain ? nullptr
                                     : (const uint32_t*)(grp.xaux + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
-            // the first loads go out before the variant flag is looked at: its load is in
-            // flight with the offsets', and nothing waits for it until the walk begins
-            TaskOpen<S, DotPolicy<BS, XM>> o;
-            open_task<S>(cur, lut, pol, id.t1 - id.t0, stage_all, o);
+            // looked at only now: the flag's load has been in flight together with the offsets'
             const bool variant = Codec::variant_test(pin_uniform(variant_word), header);
-            if (variant) walk_task<true, S>(cur, lut, pol, id.t1 - id.t0, o);
-            else walk_task<false, S>(cur, lut, pol, id.t1 - id.t0, o);
+            if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
+            else run_task<false, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
             // Nothing is in flight at the end of a task.  Saying so keeps the compiler from
             // waiting at the top of the loop for loads that a previous pass might have left
             // behind: on the first pass that wait would be for the table, before the task's
