@@ -71,6 +71,22 @@ __device__ __forceinline__ uint32_t rebuild_pair(uint32_t e, uint32_t z) {
 __device__ __forceinline__ uint32_t rem_lo_pair(uint32_t r) { return __builtin_amdgcn_perm(r, r, 0x01010000u); }
 __device__ __forceinline__ uint32_t rem_hi_pair(uint32_t r) { return __builtin_amdgcn_perm(r, r, 0x03030202u); }
 
+// Sum over the 16 lanes that share `lane & 3` (the 16 column blocks of a step), left in every
+// lane: two rotations inside the rows of 16 lanes (DPP), then the two row-swap instructions of
+// gfx950 -- no trip through the LDS crossbar, which four dependent `__shfl_xor` would take.
+__device__ __forceinline__ float sum_over_column_blocks(float a) {
+    a += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(a), 0x124, 0xF, 0xF, false));   // row_ror:4
+    a += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(a), 0x128, 0xF, 0xF, false));   // row_ror:8
+    // v_permlane16_swap exchanges rows 1, 3 of its first operand with rows 0, 2 of the second:
+    // from two copies of `a` come [r0 r0 r2 r2] and [r1 r1 r3 r3]
+    typedef uint32_t pair_t __attribute__((ext_vector_type(2)));
+    pair_t p = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(a), false, false);
+    a = __uint_as_float(p.x) + __uint_as_float(p.y);
+    // v_permlane32_swap exchanges the upper half of the first with the lower half of the second
+    p = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(a), false, false);
+    return __uint_as_float(p.x) + __uint_as_float(p.y);
+}
+
 // A word of memory that nothing writes while the kernel runs (offsets, the format header),
 // read at a wave-uniform address: through the constant address space the compiler issues a
 // scalar load, which neither queues behind the vector loads in flight nor has to be waited
@@ -97,13 +113,17 @@ struct TaskSpan { uint32_t base, end; };
 
 __device__ __forceinline__ TaskSpan task_span(const uint32_t* __restrict__ offsets, int M, int split_k, int nc,
                                               int k, int g, int c, uint32_t total_words) {
+    // offsets[k][4 * g + c] for c < nc; the stream that follows starts at the next used slot:
+    // the group's next chunk, or slot 0 of the next group (which for the last group of a split
+    // is the first slot of the next split), or, for the very last task, the end of the stream.
+    // Both loads are issued unconditionally (the second at a clamped index), without branches.
     TaskSpan s;
-    const int G = M / kGroupRows;
-    s.base = constant_word(offsets + (size_t)k * M + kGroupRows * g + c);
-    if (c + 1 < nc)            s.end = constant_word(offsets + (size_t)k * M + kGroupRows * g + c + 1);
-    else if (g + 1 < G)        s.end = constant_word(offsets + (size_t)k * M + kGroupRows * (g + 1));
-    else if (k + 1 < split_k)  s.end = constant_word(offsets + (size_t)(k + 1) * M);
-    else                       s.end = total_words;
+    const int at = k * M + kGroupRows * g;
+    const int next = c + 1 < nc ? at + c + 1 : at + kGroupRows;
+    const int slots = split_k * M;
+    s.base = constant_word(offsets + (at + c));
+    const uint32_t e = constant_word(offsets + (next < slots ? next : slots - 1));
+    s.end = next < slots ? e : total_words;
     return s;
 }
 

@@ -639,12 +639,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
         for (int q = 0; q < NSET; ++q) {
 #pragma unroll
             for (int i = 0; i < kGroupRows; ++i) {
-                float a = pol.acc[q][i];
-                a += __shfl_xor(a, 4);
-                a += __shfl_xor(a, 8);
-                a += __shfl_xor(a, 16);
-                a += __shfl_xor(a, 32);
-                pol.acc[q][i] = a;
+                pol.acc[q][i] = sum_over_column_blocks(pol.acc[q][i]);
             }
         }
     }
