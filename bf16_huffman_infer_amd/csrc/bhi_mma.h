@@ -216,12 +216,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     for (int q = 0; q < Q; ++q) {
 #pragma unroll
         for (int i = 0; i < kGroupRows; ++i) {
-            float v = pol.acc[q][i];
-            v += __shfl_xor(v, 4);
-            v += __shfl_xor(v, 8);
-            v += __shfl_xor(v, 16);
-            v += __shfl_xor(v, 32);
-            pol.acc[q][i] = v;
+            pol.acc[q][i] = sum_over_column_blocks(pol.acc[q][i]);
         }
     }
     if (a.slices == 1) {

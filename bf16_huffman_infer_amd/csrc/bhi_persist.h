@@ -272,12 +272,7 @@ void gemv_persist_kernel(const uint16_t* __restrict__ X, const PGroup grp) {
             for (int qq = 0; qq < NSET; ++qq) {
 #pragma unroll
                 for (int i = 0; i < kGroupRows; ++i) {
-                    float a = pol.acc[qq][i];
-                    a += __shfl_xor(a, 4);
-                    a += __shfl_xor(a, 8);
-                    a += __shfl_xor(a, 16);
-                    a += __shfl_xor(a, 32);
-                    pol.acc[qq][i] = a;
+                    pol.acc[qq][i] = sum_over_column_blocks(pol.acc[qq][i]);
                 }
             }
 #pragma unroll

@@ -460,11 +460,13 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
                            const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
     __shared__ uint32_t rings[NW][kRingWords];
     __shared__ uint32_t lut[Codec::kTableWords];
-    // The table reaches LDS while the task's first loads are in flight; a wavefront without
-    // a task still copies its share and joins the barrier.
+    // The table's loads go out first and its LDS writes follow the task's own first loads; a
+    // wavefront without a task still copies its share and joins the barrier.
+    TableCopy<Codec::kTableWords, NW * kLanes> table_copy;
+    table_copy.issue(table);
     auto stage_table = [&]() {
-        load_table<Codec::kTableWords>(lut, table);
-        __syncthreads();
+        table_copy.commit(lut);
+        lds_barrier();
     };
 
     const int lane = threadIdx.x & (kLanes - 1);
@@ -660,15 +662,16 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
         }
         return;
     }
-    __syncthreads();                       // every wavefront has finished reading its ring
-    float* mine = (float*)rings[wave];     // partial sums: [set][row][batch lane]
+    // partial sums, [set][row][batch lane], go into the wavefront's own ring: nobody else
+    // reads or writes it before the barrier below
+    float* mine = (float*)rings[wave];
     if (active && lane < 4) {
 #pragma unroll
         for (int q = 0; q < NSET; ++q)
 #pragma unroll
             for (int i = 0; i < kGroupRows; ++i) mine[(q * kGroupRows + i) * 4 + lane] = pol.acc[q][i];
     }
-    __syncthreads();
+    lds_barrier();
     if (active && p == 0 && lane < 4) {
 #pragma unroll
         for (int q = 0; q < NSET; ++q) {
