@@ -272,15 +272,33 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
 
 }  // namespace bhi
 
-// K slices of a launch: enough blocks for the whole GPU where the streams allow it.
+// K slices of a launch: the divisor d of the tasks per row group that minimises a small cost
+// model, in units of steps.  A block walks (tasks per group / d) tasks and pays about six
+// steps' worth of start; with at most one block per compute unit (256) the blocks run at
+// full pace, with two 8-wavefront blocks on a unit at two thirds of it, and blocks beyond
+// what is resident at once (512 of 8 wavefronts, 256 of 16) wait for a whole round; every
+// slice adds a round trip of partial sums (two steps' worth).  The model reproduces the order
+// measured at 16 / 32 rows: 4096x12288 (6 tasks of 16 steps) 2 slices 32 us, 3 slices 33 us,
+// 6 slices 41 us, none 50 us / 3 slices 44 us, 2 slices 55 us, 6 slices 59 us;
+// 3584x18944 (4 tasks of 37 steps) 4 slices 36 us, 2 slices 42 us; 4096x4096 (4 tasks of 8
+// steps) 2 slices 17 us, 4 slices 20 us; 4608x3584 2 slices 20 / 29 us, 4 slices 24 / 42 us.
 static inline int mma_slices(const bhi::Shape& s, int nw) {
     using namespace bhi;
     const int G = s.M / kGroupRows, per_group = s.split_k * s.nc;
     if (G >= kMmaSliceBelowGroups) return 1;
-    const long long want = 256 * (16 / nw);                  // row blocks x slices: all compute units busy
+    const long long row_blocks = G / nw;
+    const double task_steps = (double)s.steps / s.nc;
     int best = 1;
-    for (int d = 1; d <= kMmaMaxSlices && d <= per_group; ++d)
-        if (per_group % d == 0 && (long long)(G / nw) * best < want) best = d;
+    double best_cost = 0;
+    for (int d = 1; d <= kMmaMaxSlices && d <= per_group; ++d) {
+        if (per_group % d != 0) continue;
+        const long long blocks = row_blocks * d;
+        double pace;
+        if (nw <= 8) pace = blocks <= 256 ? 1.0 : 1.5 * (double)((blocks + 511) / 512);
+        else pace = (double)((blocks + 255) / 256);
+        const double cost = pace * (per_group / d * task_steps + 6.0) + 2.0 * d;
+        if (d == 1 || cost < best_cost) { best = d; best_cost = cost; }
+    }
     return best;
 }
 

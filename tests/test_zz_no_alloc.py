@@ -46,12 +46,12 @@ def test_static_workspace_entry_matches_the_workspace_entry(cuda):
 
 
 def test_static_workspace_entry_rejects_what_does_not_fit(cuda):
-    """8064 x 28672 at 32 rows is cut into 4 K slices: 4.1 MB of partial sums, twice what
-    the built-in workspace holds.  The entry point says so before it touches any buffer (the
-    pointers given here are placeholders)."""
+    """6400 x 12288 (three splits of 4096 columns) at 32 rows is cut into 3 K slices: 2.46 MB of
+    partial sums, more than the built-in workspace holds.  The entry point says so before it
+    touches any buffer (the pointers given here are placeholders)."""
     from bf16_huffman_infer_amd import _lib
     lib = _lib.load()
-    M, split_k, Ks, rows = 8064, 8, 3584, 32
+    M, split_k, Ks, rows = 6400, 3, 4096, 32
     need = lib.bhi_gemm_workspace_bytes(split_k, M, Ks, rows)
     assert need > lib.bhi_gemm_static_workspace_bytes() == 1024 + (2 << 20)
     dummy = torch.zeros(4096, dtype=torch.int32, device="cuda")
