@@ -155,3 +155,33 @@ def test_get_model_size_counts_parameters_and_buffers():
     lin = CompressedLinear(_huffman_weight(128, 384), torch.nn.Parameter(torch.ones(128).bfloat16(), requires_grad=False))
     want = sum(b.nelement() * b.element_size() for b in lin.weight.buffers()) + 128 * 2
     assert get_model_size(lin) == want == 128 * 384 + (32 * 64 + 2048) * 4 + 128 * 4 + 8192 + 4 * 256 + 256
+
+
+def test_workspace_of_the_fused_product_follows_the_slice_choice():
+    """`bhi_gemm_workspace_bytes` is host arithmetic: 1 KiB of arrival counters plus
+    slices x rows x M floats, nothing for a weight that is not cut along K.  The slice counts
+    are the ones measured fastest on the GPU for these shapes."""
+    from bf16_huffman_infer_amd import _lib
+    lib = _lib.load()
+
+    def slices(split_k, M, Ks, rows):
+        need = lib.bhi_gemm_workspace_bytes(split_k, M, Ks, rows)
+        if need == 0:
+            return 1
+        assert (need - 1024) % (rows * M * 4) == 0
+        return (need - 1024) // (rows * M * 4)
+
+    assert slices(1, 12288, 4096, 16) == 1 and slices(1, 12288, 4096, 32) == 1      # 3072 row groups: never cut
+    assert slices(3, 4096, 4096, 16) == 2 and slices(3, 4096, 4096, 32) == 3        # 4096x12288, 6 tasks per group
+    assert slices(4, 3584, 4736, 16) == 4 and slices(4, 3584, 4736, 32) == 4        # 3584x18944, 4 long tasks
+    assert slices(1, 4096, 4096, 16) == 2 and slices(1, 4608, 3584, 16) == 2
+    # every choice divides the tasks of a row group, and the built-in workspace holds whatever
+    # stays within one block per compute unit
+    static = lib.bhi_gemm_static_workspace_bytes()
+    for split_k, M, Ks in [(1, 1024, 4096), (2, 2048, 2048), (8, 4096, 1024), (3, 4096, 4096), (1, 8128, 3584)]:
+        per_group = split_k * lib.bhi_chunks_per_group(M, Ks, split_k)
+        for rows in (9, 16, 17, 32):
+            d = slices(split_k, M, Ks, rows)
+            assert per_group % d == 0
+            if (M // 4 // (8 if rows <= 16 else 16)) * d <= 256:
+                assert lib.bhi_gemm_workspace_bytes(split_k, M, Ks, rows) <= static
