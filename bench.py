@@ -31,10 +31,12 @@ STD = 0.02
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this script, each scaled by the same counter's reading for the 256 MiB calibration
 # copy below.  Keyed by (algo, batch, launch): "single" = one 18944x3584 matrix, "group" =
-# gate_proj + up_proj in one launch.  The readings belong to the kernel sources whose digest
-# is recorded with them: when the sources have changed since, `traffic` is reported as null.
+# gate_proj + up_proj in one launch, "lm_head" = the 152064x3584 launch.  The readings belong
+# to the kernel sources whose digest is recorded with them: when the sources have changed
+# since, `traffic` is reported as null.
 MEASURED_TRAFFIC_SOURCES = "d6e09bd55f88d1bf"
-MEASURED_TRAFFIC = {("huffman", 1, "single"): 94880000, ("huffman", 1, "group"): 200820000}
+MEASURED_TRAFFIC = {("huffman", 1, "single"): 94880000, ("huffman", 1, "group"): 200820000,
+                    ("huffman", 1, "lm_head"): 809560000}
 
 
 def kernel_sources_digest() -> str:
@@ -79,6 +81,37 @@ def build_block(algo, device, copy):
             mods.append(cls[algo].compress(w).to(device))
         del w
     return mods
+
+
+LM_HEAD = (152064, 3584)      # the model's largest linear: vocabulary x hidden
+
+
+def lm_head(args, device):
+    """The same kernel on the model's lm_head, one launch of 38016 tasks (six times what the
+    GPU holds at once), so that launch, first fill and the last blocks weigh little: what the
+    kernel sustains when a launch is long enough.  Two clones alternate (375 MB each, more
+    than the 256 MB last-level cache)."""
+    import copy
+    import torch.nn.functional as F
+    from bf16_huffman_infer_amd.functional import ANSWeight, HuffmanWeight, NibbleWeight
+    M, K = LM_HEAD
+    cls = {"huffman": HuffmanWeight, "ans": ANSWeight, "nibble": NibbleWeight}[args.algo]
+    w = make_weight(M, K, 77, device)
+    mod = cls.compress(w).to(device)
+    del w
+    mods = [mod, copy.deepcopy(mod)]
+    x = torch.randn(args.batch, K, device=device).bfloat16()
+    st = {"i": 0}
+
+    def one():
+        F.linear(x, mods[st["i"] % 2])
+        st["i"] += 1
+    t = time_launches(one, max(60, args.steps // 2), args.warmup, launches_per_graph=2)
+    nbytes = gemv_bytes(mod, args.batch, M, K)
+    return {"shape": f"{M}x{K}", "tasks": M // 4, "bytes_per_launch": nbytes, "us_per_launch": round(t * 1e6, 2),
+            "achieved": round(nbytes / t / 1e9, 1), "frac": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": measured_traffic((args.algo, args.batch, "lm_head")),
+            "compression_ratio": round(weight_bytes(mod) / (2 * M * K), 4)}
 
 
 def sweep(args, device, huffman_blocks):
@@ -238,6 +271,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the other batches / codecs")
     ap.add_argument("--no-fallback", action="store_true", help="skip the 16- and 32-row fused matrix product")
     ap.add_argument("--no-decode", action="store_true", help="skip the 36-layer decoder (tokens/s)")
+    ap.add_argument("--no-lm-head", action="store_true", help="skip the 152064x3584 launch")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1")
@@ -373,6 +407,9 @@ def main():
         out["sweep"] = sweep(args, device, blocks)
     del blocks
     torch.cuda.empty_cache()
+    if not args.no_lm_head:
+        out["lm_head"] = lm_head(args, device)
+        torch.cuda.empty_cache()
     if not args.no_fallback:
         # more than 8 rows of X: the fused decode + matrix-core product beside decode-to-BF16 + dense GEMM
         from bench_fallback import measure
