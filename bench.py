@@ -153,11 +153,15 @@ def sweep(args, device, huffman_blocks):
     return out
 
 
-def time_launches(fn, n, warmup, launches_per_graph=1):
-    """Seconds per call of ``fn``.  ``fn`` is captured once into a HIP graph (as the decode
-    step is in serving, and as the reference's own benchmark does with CUDA graphs) so
-    that the Python dispatch cost of the op wrappers is not what gets timed; the graph
-    holds ``launches_per_graph`` consecutive calls."""
+ROUNDS = 5
+
+
+def time_launches(fn, n, warmup, launches_per_graph=1, rounds=ROUNDS, spread=None):
+    """Seconds per call of ``fn``: the median of ``rounds`` timed regions of ``n`` calls each.
+    ``fn`` is captured once into a HIP graph (as the decode step is in serving, and as the
+    reference's own benchmark does with CUDA graphs) so that the Python dispatch cost of the
+    op wrappers is not what gets timed; the graph holds ``launches_per_graph`` consecutive
+    calls.  ``spread``, a dict, receives the fastest and the slowest round."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -187,12 +191,18 @@ def time_launches(fn, n, warmup, launches_per_graph=1):
     for _ in range(int(CLOCK_WARMUP_S / once) + 1):
         graph.replay()
     torch.cuda.synchronize()
-    start.record()
-    for _ in range(replays):
-        graph.replay()
-    stop.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(stop) * 1e-3 / (replays * launches_per_graph)
+    times = []
+    for _ in range(max(1, rounds)):
+        start.record()
+        for _ in range(replays):
+            graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(stop) * 1e-3 / (replays * launches_per_graph))
+    times.sort()
+    if spread is not None:
+        spread.update(rounds=len(times), calls_per_round=replays * launches_per_graph, min=times[0], max=times[-1])
+    return times[len(times) // 2]
 
 
 def load_only(launch_bytes, args, device):
@@ -320,8 +330,10 @@ def main():
         linear_grouped(xs[2], [mods[2], mods[3]])
         F.linear(xs[4], mods[4])
 
-    sec_single = time_launches(step_single, args.steps, args.warmup, launches_per_graph=COPIES)
-    sec = sec_single if args.no_group else time_launches(step_grouped, args.steps, args.warmup, launches_per_graph=COPIES)
+    spread = {}
+    sec_single = time_launches(step_single, args.steps, args.warmup, launches_per_graph=COPIES, spread=spread)
+    sec = sec_single if args.no_group else time_launches(step_grouped, args.steps, args.warmup, launches_per_graph=COPIES,
+                                                         spread=spread)
     gbs = block_bytes / sec / 1e9
 
     # Per-layer timing and the roofline of the dominant kernel.  A layer alone must not be
@@ -377,6 +389,9 @@ def main():
                                f"down 3584x18944), N(0,0.02) seeded, algo={args.algo}, batch={bs}, {COPIES} "
                                f"alternating weight copies, "
                                f"{'5 launches' if args.no_group else '4 launches (gate+up grouped)'} per step"},
+        # ms_per_step is the median of this many timed regions of --steps steps; fastest and slowest beside it
+        "ms_per_step_rounds": {"rounds": spread["rounds"], "steps_per_round": spread["calls_per_round"],
+                               "min": round(spread["min"] * 1e3, 5), "max": round(spread["max"] * 1e3, 5)},
         "clock_warmup_ms": CLOCK_WARMUP_S * 1e3,   # untimed replays before every timed region, on top of --warmup
         "ms_per_step_single_launches": round(sec_single * 1e3, 5),
         "pct_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
@@ -413,7 +428,7 @@ def main():
     if not args.no_fallback:
         # more than 8 rows of X: the fused decode + matrix-core product beside decode-to-BF16 + dense GEMM
         from bench_fallback import measure
-        out["fallback"] = measure(device, with_library_gemm=False, steps=max(50, args.steps // 2))
+        out["fallback"] = measure(device, with_library_gemm=True, steps=max(50, args.steps // 2))
         torch.cuda.empty_cache()
     if not args.no_decode:
         # the tokens/s half of the metric, measured: Qwen3-8B-shaped decoder, 36 layers, algo=smallest,
@@ -423,7 +438,7 @@ def main():
         torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
-    print(json.dumps(out))
+    print(json.dumps(out, allow_nan=False))
 
 
 if __name__ == "__main__":

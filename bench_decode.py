@@ -378,7 +378,7 @@ def run(args) -> dict:
 
 
 def main():
-    print(json.dumps(run(parse_args())))
+    print(json.dumps(run(parse_args()), allow_nan=False))
 
 
 if __name__ == "__main__":

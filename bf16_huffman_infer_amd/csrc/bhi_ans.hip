@@ -17,7 +17,6 @@ constexpr int kAnsInitRows = 2;                 // rows 0, 1 of a lane: its init
 struct AnsCodec {
     using Cursor = AnsCursor;
     static constexpr bool kTransformsX = true;    // kernels with RMSNorm / SiLU*mul in front of the product are built
-    static constexpr bool kPersistent = true;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = kAnsTableWords;
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__) { return false; }
     static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__) { return 0u; }

@@ -13,7 +13,6 @@ namespace bhi {
 struct HuffCodec {
     using Cursor = HuffCursor;
     static constexpr bool kTransformsX = true;    // kernels with RMSNorm / SiLU*mul in front of the product are built
-    static constexpr bool kPersistent = true;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = kTableEntries;
     // escaped pairs need the slower walk; the header says whether the matrix has any
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ header) { return header_has_esc(header); }

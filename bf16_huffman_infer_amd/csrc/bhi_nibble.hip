@@ -15,7 +15,6 @@ constexpr uint32_t kNibbleEsc = 15;
 struct NibbleCodec {
     using Cursor = NibbleCursor;
     static constexpr bool kTransformsX = false;    // kernels with RMSNorm / SiLU*mul in front of the product are built
-    static constexpr bool kPersistent = false;     // whether the persistent grid can walk this codec
     static constexpr int kTableWords = 4;          // base and flags, one 16-byte copy
     static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__ lut) {
         return constant_word((const uint32_t*)lut + 1);

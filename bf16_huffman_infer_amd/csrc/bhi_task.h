@@ -80,11 +80,11 @@ __device__ __forceinline__ void decode_segment(Cursor& cur, const uint32_t* lut,
 template <bool HAS_ESC, int S, class Cursor, class Policy>
 __device__ __forceinline__ void run_segment(Cursor& cur, const uint32_t* lut, Policy& pol, bool& pending,
                                             uint32_t (&rows)[S], const typename Policy::Slot (&now)[S],
-                                            typename Policy::Slot (&next)[S], int seg, int next_seg, int ns) {
+                                            typename Policy::Slot (&next)[S], int seg, int next_seg, bool spare, int ns) {
     if (pending) cur.commit(rows);
     pending = cur.template room<S>();
     if (pending) cur.prefetch(rows);
-    pol.load_full(next, next_seg);
+    pol.load_full(next, next_seg, spare);
     decode_segment<true, HAS_ESC>(cur, lut, pol, now, seg, ns);
 }
 
@@ -101,7 +101,7 @@ __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Polic
     const int last_full = full_end - S;
     pol.prime();
     if (full_end > 0) {
-        pol.load_full(a, 0);
+        pol.load_full(a, 0, false);
     } else {
 #pragma unroll
         for (int i = 0; i < S; ++i) pol.load(a[i], i);
@@ -120,11 +120,11 @@ __device__ __forceinline__ void run_task(Cursor& cur, const uint32_t* lut, Polic
     if (full_end > 0) {
         for (;;) {
             int nx = seg + S;
-            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, ns);
+            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, a, b, seg, nx < last_full ? nx : last_full, nx > last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
             nx = seg + S;
-            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, ns);
+            run_segment<HAS_ESC, S>(cur, lut, pol, pending, rows, b, a, seg, nx < last_full ? nx : last_full, nx > last_full, ns);
             seg = nx;
             if (seg >= full_end) break;
         }
@@ -173,7 +173,7 @@ struct StorePolicy {
         s.rem = stream_load(rem0 + (size_t)t * kLanes);
     }
     template <int S>
-    __device__ __forceinline__ void load_full(Slot (&s)[S], int t0) const {
+    __device__ __forceinline__ void load_full(Slot (&s)[S], int t0, bool) const {
         const uint2* p = rem0 + (size_t)t0 * kLanes;
 #pragma unroll
         for (int i = 0; i < S; ++i) s[i].rem = stream_load(p + i * kLanes);
@@ -341,6 +341,7 @@ struct DotPolicy {
     struct Slot { uint2 rem; uint4 x; uint4 a; };            // x: the lane's X pair of batch rows 0..3; a: gamma or gate pairs
     struct Piped { uint4 x, a; int i, t; };
     const uint2* rem0;
+    const uint2* spare_rem;  // kSegLong * 512 readable bytes that are cache resident (the decode table, or the task's start)
     const uint32_t* xq0;     // this lane's X pair of batch row 0, first step of the task
     const uint32_t* aq0;     // the same position in gamma (kXRms) or in gate row 0 (kXSiluMul)
     float rs[BS <= 4 ? BS : 1];   // kXRms: the rows' scales
@@ -379,9 +380,11 @@ struct DotPolicy {
         if (XM == kXRms) s.a.x = a0[(size_t)t * (kStepCols / 2)];
         if (XM == kXSiluMul) xpairs<0>(s.a, a0 + (size_t)t * (kStepCols / 2));
     }
+    // `spare`: the loads are not needed (the last whole segment of a task has no successor) and
+    // go to `spare_rem`, bytes that are in cache anyway, instead of reading the segment again
     template <int S>
-    __device__ __forceinline__ void load_full(Slot (&s)[S], int t0) const {
-        const uint2* pr = rem0 + (size_t)t0 * kLanes;
+    __device__ __forceinline__ void load_full(Slot (&s)[S], int t0, bool spare) const {
+        const uint2* pr = spare ? spare_rem : rem0 + (size_t)t0 * kLanes;
         const uint32_t* pq = xq0 + (size_t)t0 * (kStepCols / 2);
         const uint32_t* pa = aq0 + (size_t)t0 * (kStepCols / 2);
 #pragma unroll
@@ -625,6 +628,7 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
             pol.aq0 = XM == kXPlain ? nullptr
                                     : (const uint32_t*)(grp.xaux + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
+            pol.spare_rem = Codec::kTableWords * 4 >= kSegLong * kLanes * 8 ? (const uint2*)table + lane : pol.rem0;
             // looked at only now: the flag's load has been in flight together with the offsets'
             const bool variant = Codec::variant_test(pin_uniform(variant_word), header);
             if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
@@ -691,8 +695,6 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
 
 }  // namespace bhi
 
-#include "bhi_persist.h"
-
 static inline int check_shape(int split_k, int M, int Ks, int64_t exp_words, bhi::Shape* s) {
     using namespace bhi;
     if (split_k < 1 || M < kGroupRows || M % kGroupRows != 0 || Ks < kStepCols || Ks % kStepCols != 0)
@@ -758,11 +760,6 @@ static inline void launch_gemv_batch(int batch, const void* X, const bhi::Group&
     if constexpr (Codec::kTransformsX) {
         if (x_mode == bhi::kXRms) return launch_gemv_x<Codec, bhi::kXRms>(batch, X, grp, blocks, st);
         if (x_mode == bhi::kXSiluMul) return launch_gemv_x<Codec, bhi::kXSiluMul>(batch, X, grp, blocks, st);
-    }
-    if constexpr (Codec::kPersistent) {
-        bool plain = true;
-        for (int i = 0; i < grp.n; ++i) plain = plain && !grp.m[i].residual;
-        if (plain && try_launch_persist<Codec>(batch, X, grp, st)) return;
     }
     switch (batch) {
         case 1: launch_gemv<Codec, 1>(X, grp, blocks, st); break;

@@ -57,3 +57,27 @@ def test_reference_ans_buffers_decode_and_transcode(cuda, maker, split_k):
     assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), bits)
     mine = transcode_reference_weight(buffers, algo="smallest").cuda()
     assert torch.equal(mine.get_weight().cpu().view(torch.int16), w.view(torch.int16))
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("K,split_k", [(384, 1), (768, 2)])
+def test_reference_buffers_of_several_parts(cuda, K, split_k, algo):
+    """8320 rows: three 4096-row parts per split, each followed by its 64 zero words, offsets
+    running on across parts and splits (reference ``functional.py:202-231``) -- the shape of
+    every layer of a real checkpoint."""
+    from bf16_huffman_infer_amd.reference_format import (decode_reference_ans, decode_reference_huffman,
+                                                         transcode_reference_weight)
+    from test_oracle_cpu import multi_part_case
+    bits, enc, tables, _ = multi_part_case(K, split_k, algo)
+    buffers = dict(rem=_t(enc["rem"]), exp=_t(enc["exp"]), offsets=_t(enc["offsets"]))
+    if algo == "huffman":
+        luts, lens = tables
+        buffers.update(LUT1=_t(luts[0]), LUT2=_t(luts[1]), LUT3=_t(luts[2]), LUT4=_t(luts[3]), code_lengths=_t(lens))
+        got = decode_reference_huffman(**buffers)
+    else:
+        buffers.update(LUT=_t(tables[0]))
+        got = decode_reference_ans(**buffers)
+    assert np.array_equal(got.cpu().view(torch.int16).numpy().view(np.uint16), bits)
+    mine = transcode_reference_weight(buffers).cuda()
+    assert type(mine).__name__ == ("HuffmanWeight" if algo == "huffman" else "ANSWeight")
+    assert np.array_equal(mine.get_weight().cpu().view(torch.int16).numpy().view(np.uint16), bits)

@@ -121,6 +121,51 @@ def test_reference_layout_round_trip(maker, M, K, split_k):
     assert np.array_equal(ref_layout.decode_ans(enc["rem"], enc["exp"], enc["offsets"], lut), bits)
 
 
+def multi_part_case(K, split_k, algo, seed=6):
+    """8320 rows = two whole parts of 4096 and one of 128, as every layer of a real model has
+    (reference ``functional.py:202-209``).  Returns (bits, encoded buffers, decode tables)."""
+    bits = bits_of(gaussian_weight(8320, K, seed=seed))
+    _, exp = planes.split_bf16(bits)
+    counts = np.bincount(exp.reshape(-1), minlength=256)
+    if algo == "huffman":
+        luts, lens, codes = ref_tables.build_cascade_luts(counts)
+        return bits, ref_layout.encode(bits, split_k, "huffman", codes), (luts, lens), codes
+    freq, cum, lut = ref_tables.ans_tables(counts)
+    return bits, ref_layout.encode(bits, split_k, "ans", (freq, cum)), (lut,), (freq, cum)
+
+
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("K,split_k", [(384, 1), (768, 1), (768, 2)])
+def test_reference_layout_parts_pads_and_rebased_offsets(K, split_k, algo):
+    """Several 4096-row parts per split: 64 zero words behind every part (reference
+    ``functional.py:177``), offsets running on across parts and splits (``:210-231``), and a part's
+    words independent of what surrounds it."""
+    bits, enc, tables, enc_tables = multi_part_case(K, split_k, algo)
+    M, Ks = bits.shape[0], K // split_k
+    exp, off = enc["exp"].view(np.uint32), enc["offsets"].astype(np.int64)
+    part_starts = [0, 4096, 8192]
+    assert off[0, 0] == 0 and (np.diff(off.reshape(-1)) > 0).all()
+    ends = np.append(off.reshape(-1)[1:], exp.size)                  # where the next row (or the stream) begins
+    for k in range(split_k):
+        for j, r0 in enumerate(part_starts):
+            r1 = min(r0 + 4096, M)
+            # the part's rows are followed by exactly one row of 64 zero words, which belongs to no row
+            part_end = ends[k * M + r1 - 1]
+            assert not exp[part_end - 64:part_end].any()
+            row_words = np.diff(np.append(off[k, r0:r1], part_end - 64))
+            assert (row_words % 64 == 0).all() and (row_words > 0).all()
+            # the same rows compressed on their own: the same words, offsets shifted by the part's base
+            alone = ref_layout.encode(bits[r0:r1, k * Ks:(k + 1) * Ks], 1, algo, enc_tables)
+            assert np.array_equal(alone["exp"].view(np.uint32), exp[off[k, r0]:part_end])
+            assert np.array_equal(alone["offsets"][0].astype(np.int64) + off[k, r0], off[k, r0:r1])
+    assert ends[-1] == exp.size
+    if algo == "huffman":
+        got = ref_layout.decode_huffman(enc["rem"], enc["exp"], enc["offsets"], *tables)
+    else:
+        got = ref_layout.decode_ans(enc["rem"], enc["exp"], enc["offsets"], *tables)
+    assert np.array_equal(got, bits)
+
+
 def test_reference_cascade_hole_is_real():
     """The reference reserves 255 as the miss marker, so exponent 255 (inf/NaN) cannot be
     told from a miss; recorded here so nobody trusts the cascade on such tensors."""
