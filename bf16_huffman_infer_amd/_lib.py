@@ -54,9 +54,17 @@ _SIGNATURES = {
     "bhi_gemm_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "bhi_gemm_bf16_huffman_static": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp]),
     "bhi_gemm_static_workspace_bytes": (_i64, []),
+    "bhi_device_init": (_i32, []),
+    "bhi_gemm_workspace_reset": (_i32, [_vp, _i64, _vp]),
     "bhi_reference_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "bhi_reference_ans_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
 }
+
+_CONST_NAMES = (
+    "format_version", "lanes", "group_rows", "step_cols", "table_bits", "window_words",
+    "header_bits", "max_batch", "ans_precision", "align_words", "tail_pad_words",
+    "target_tasks", "max_task_steps", "member_bytes",
+)
 
 EXPORTS = tuple(_SIGNATURES)
 
@@ -75,6 +83,11 @@ def load() -> ctypes.CDLL:
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = res, args
+        buf = (ctypes.c_int32 * len(_CONST_NAMES))()
+        if lib.bhi_constants(buf, len(_CONST_NAMES)) != len(_CONST_NAMES):
+            raise RuntimeError("constant table of the library and of the binding differ: rebuild the library")
+        if buf[_CONST_NAMES.index("member_bytes")] != ctypes.sizeof(GemvMember):
+            raise RuntimeError("bhi_gemv_member of the library and of the binding differ: rebuild the library")
         _lib = lib
     return _lib
 
@@ -83,13 +96,6 @@ def check(rc: int, what: str) -> None:
     if rc != 0:
         msg = load().bhi_last_error_string().decode()
         raise RuntimeError(f"{what} failed (code {rc}): {msg}")
-
-
-_CONST_NAMES = (
-    "format_version", "lanes", "group_rows", "step_cols", "table_bits", "window_words",
-    "header_bits", "max_batch", "ans_precision", "align_words", "tail_pad_words",
-    "target_tasks", "max_task_steps",
-)
 
 
 def constants() -> dict:

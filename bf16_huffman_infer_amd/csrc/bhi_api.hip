@@ -23,6 +23,7 @@ extern "C" int bhi_constants(int32_t* out, int n) {
         bhi::kFormatVersion, bhi::kLanes, bhi::kGroupRows, bhi::kStepCols, bhi::kTableBits,
         bhi::kWindowWords, bhi::kHeaderBits, bhi::kMaxBatch, bhi::kAnsPrecision,
         bhi::kAlignWords, bhi::kTailPadWords, bhi::kTargetTasks, bhi::kMaxTaskSteps,
+        (int32_t)sizeof(bhi_gemv_member),
     };
     const int total = (int)(sizeof(v) / sizeof(v[0]));
     for (int i = 0; out && i < n && i < total; ++i) out[i] = v[i];
@@ -135,4 +136,26 @@ extern "C" int bhi_silu_mul(const void* gate, const void* up, void* out, int64_t
     hipLaunchKernelGGL(bhi::silu_mul_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                        (const uint32_t*)gate, (const uint32_t*)up, (uint32_t*)out, pairs);
     return bhi_launch_status("silu_mul");
+}
+
+// ---------------------------------------------------------------------------------------------
+// A workspace of the fused matrix product back to the state the library expects (all zero): for
+// a caller whose launch failed or was abandoned halfway, where counters may be left non-zero.
+// A fill kernel, not a memset: it may be recorded into a graph.
+namespace bhi {
+__global__ __launch_bounds__(256) void zero_kernel(uint32_t* __restrict__ p, long long words) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (long long)gridDim.x * blockDim.x) p[i] = 0u;
+}
+}  // namespace bhi
+
+extern "C" int bhi_gemm_workspace_reset(void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!workspace || workspace_bytes < 0 || workspace_bytes % 4 != 0 || ((uintptr_t)workspace & 3) != 0)
+        return bhi_fail(BHI_EINVAL, "workspace must be a 4-byte aligned region of whole words");
+    const long long words = workspace_bytes / 4;
+    if (words > 0) {
+        const long long blocks = (words + 255) / 256;
+        hipLaunchKernelGGL(bhi::zero_kernel, dim3((unsigned)(blocks < 1024 ? blocks : 1024)), dim3(256), 0, (hipStream_t)stream,
+                           (uint32_t*)workspace, words);
+    }
+    return bhi_launch_status("gemm_workspace_reset");
 }

@@ -192,6 +192,14 @@ extern "C" int bhi_gemm_bf16_huffman_static(const bhi_gemv_member* weight, const
 
 extern "C" int64_t bhi_gemm_static_workspace_bytes(void) { return kStaticWorkspaceBytes; }
 
+// Everything the library looks up once per device (today: the address of the built-in
+// workspace), looked up now, on the current device: a caller that will first use the library
+// under stream capture calls this beforehand, outside the capture.
+extern "C" int bhi_device_init(void) {
+    void* ws = nullptr;
+    return static_workspace(&ws);
+}
+
 extern "C" int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch) {
     Shape s;
     if (batch < 1 || batch > kMmaMaxBatch) return bhi_fail(BHI_EBATCH, "the fused matrix product takes 1 to 32 rows of X");

@@ -40,6 +40,12 @@ namespace bhi {
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
+#ifndef BHI_MMA_ARRIVAL_ORDER
+#define BHI_MMA_ARRIVAL_ORDER __ATOMIC_RELAXED
+#endif
+#ifndef BHI_MMA_LAST_ACQUIRES
+#define BHI_MMA_LAST_ACQUIRES 1
+#endif
 constexpr int kMmaSeg = 4;                   // steps per window
 // wavefronts (row groups) per block: LDS holds two windows of X (8 KB per batch quad) beside
 // the table and the rings; up to 16 rows two 8-wavefront blocks fit a compute unit, above
@@ -233,10 +239,18 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
         }
         return;
     }
-    // ---- K slices: this block's sums go to the workspace with device-scope stores (they
-    // pass the L2 of this die, which the other dies do not see); once they have been
-    // acknowledged the block arrives at its row block's counter.  No cache-wide write-back
-    // or invalidation: with 6144 wavefronts doing one each the launch took 270 us.
+    // ---- K slices: this block's sums go to the workspace with agent-scope stores: they are
+    // written through the L2 of this die (which the other dies do not see) to the memory side
+    // all dies share, and `s_waitcnt vmcnt(0)` returns once they have been acknowledged there.
+    // Then the block arrives at its row block's counter.  The last block to arrive executes ONE
+    // agent-scope acquire (thread 0; the barrier behind it carries the order to the other
+    // threads) before it reads the other blocks' sums.  The arrival itself is a relaxed atomic:
+    // a release there makes every arriving block write back its die's whole L2, which holds
+    // nothing of this kernel that is not written through already, and costs 2.5-2.9 us of a
+    // 17-32 us launch (measured: 4096x12288 at 16 rows 31.9 -> 34.5 us, 4096x4096 16.7 -> 19.4 us;
+    // the acquire in the last block: +0.1-0.4 us).  A cache-wide fence per WAVEFRONT, 6144 of
+    // them, made the launch take 270 us.  What this relies on beyond the language's memory model:
+    // an acknowledged agent-scope store is visible to agent-scope loads of every die.
     if (lane < 4) {
 #pragma unroll
         for (int q = 0; q < Q; ++q) {
@@ -252,8 +266,9 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the stores above have completed
     __syncthreads();
     if (threadIdx.x == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(a.counters + rb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t old = __hip_atomic_fetch_add(a.counters + rb, 1u, BHI_MMA_ARRIVAL_ORDER, __HIP_MEMORY_SCOPE_AGENT);
         is_last = old == (uint32_t)a.slices - 1;
+        if (BHI_MMA_LAST_ACQUIRES && is_last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
     __syncthreads();
     if (!is_last) return;

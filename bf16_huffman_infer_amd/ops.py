@@ -34,8 +34,20 @@ _EXTRA.define("nibble_decode(Tensor A_rem, Tensor A_exp, Tensor(a!) Y, Tensor of
 LANE_BYTES_PER_STEP = 512          # 64 lanes x 8 exponent bytes
 
 
+_ready_devices = set()
+
+
 def _stream(t: Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    """The current torch stream of ``t``'s device.  The first op on a device also lets the
+    library do its once-per-device lookups: whatever comes first in a process is an eager call
+    (a conversion, a warm-up), so none of them is left for a call under stream capture."""
+    device = t.device
+    if device not in _ready_devices:
+        if not torch.cuda.is_current_stream_capturing():
+            with torch.cuda.device(device):
+                _lib.check(_lib.load().bhi_device_init(), "device_init")
+            _ready_devices.add(device)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _req(t: Tensor, dtype, name: str, ref: Tensor = None) -> int:
@@ -396,20 +408,21 @@ def _fill_member(m, w, Y: Tensor, bias, ref: Tensor) -> bool:
 
 
 GEMM_MAX_ROWS = 32
-_workspaces = {}          # device -> zero-initialised uint8 tensor; every launch leaves its counters at zero
+_workspaces = {}          # (device, stream) -> [zero-initialised uint8 tensors]; every launch leaves its counters at zero
 
 
-def _gemm_workspace(device: torch.device, nbytes: int) -> Tensor:
-    """The fused matrix product's workspace on ``device``: partial sums of K slices and the
-    arrival counters of their row blocks.  One per device, reused by every call, so calls that
-    overlap on one GPU (different streams) must not share a device's workspace -- as with any
-    library workspace.  Grown by replacement; the old one is kept alive because enqueued
-    launches may still use it."""
-    held = _workspaces.get(device)
+def _gemm_workspace(device: torch.device, stream: int, nbytes: int, allocate=None) -> Tensor:
+    """The fused matrix product's workspace for launches on ``stream`` of ``device``: partial
+    sums of K slices and the arrival counters of their row blocks.  One per (device, stream):
+    launches on one stream run one after the other and may share it, launches on different
+    streams may overlap and must not.  Grown by replacement; the old one is kept alive because
+    enqueued launches may still use it."""
+    key = (device, stream)
+    held = _workspaces.get(key)
     if held is None or held[-1].numel() < nbytes:
-        fresh = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[device] = (held or []) + [fresh]
-        held = _workspaces[device]
+        make = allocate or (lambda n: torch.zeros(n, dtype=torch.uint8, device=device))
+        _workspaces[key] = (held or []) + [make(max(nbytes, 1 << 20))]
+        held = _workspaces[key]
     return held[-1]
 
 
@@ -419,10 +432,13 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
 
     Takes the place of ``get_weight()`` + ``F.linear`` in the reference's path above eight
     rows (``functional.py:405-407, 460-462``).  ``X`` bf16 ``[rows, split_k, Ks]``, ``Y`` bf16
-    ``[rows, M]`` written.  Plain function: only enqueues on the current stream.  The first call
-    on a device allocates the workspace; when that call happens under stream capture, where
-    nothing may be allocated, a Huffman weight goes through the entry point that uses the
-    library's built-in workspace instead."""
+    ``[rows, M]`` written.  Plain function: only enqueues on the current stream.  Products that
+    are cut along K keep their partial sums in a workspace that belongs to the (device, stream)
+    pair of the call, allocated at the first such call.  Under stream capture nothing may be
+    allocated: a call that finds no workspace for the capturing stream goes, for a Huffman
+    weight, through the entry point that uses the array built into the library -- ONE array per
+    GPU, shared by every graph captured that way, so replays of two such graphs that overlap on
+    the GPU race; call once on the stream outside the capture to give it a workspace of its own."""
     lib = _lib.load()
     split_k, M, Ks = _weight_dims(weight.rem, weight.offsets)
     if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
@@ -435,20 +451,27 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
     huffman = _fill_member(member[0], weight, Y, bias, weight.rem)
     name = "gemm_bf16_huffman" if huffman else "gemm_bf16_ans"
     device = weight.rem.device
+    stream = _stream(weight.rem)
     with torch.cuda.device(device):
         need = int(lib.bhi_gemm_workspace_bytes(split_k, M, Ks, rows))
         if need < 0:
             _lib.check(need, name)
-        held = _workspaces.get(device)
-        if (held is None or held[-1].numel() < need) and torch.cuda.is_current_stream_capturing():
+        held = _workspaces.get((device, stream))
+        ws = None
+        if need == 0:
+            rc = getattr(lib, "bhi_" + name)(member, x_ptr, split_k, Ks, rows, None, 0, stream)
+        elif (held is None or held[-1].numel() < need) and torch.cuda.is_current_stream_capturing():
             # nothing may be allocated under capture: the library's built-in workspace serves
-            if not huffman or need > int(lib.bhi_gemm_static_workspace_bytes()):
-                raise RuntimeError("gemm_bf16: no workspace on this device yet and the stream is capturing; "
-                                   "call once outside the capture first")
-            rc = lib.bhi_gemm_bf16_huffman_static(member, x_ptr, split_k, Ks, rows, _stream(weight.rem))
+            if not huffman or need > int(lib.bhi_gemm_static_workspace_bytes()) or device not in _ready_devices:
+                raise RuntimeError("gemm_bf16: no workspace for this stream yet and the stream is capturing; "
+                                   "call once on this stream outside the capture first")
+            rc = lib.bhi_gemm_bf16_huffman_static(member, x_ptr, split_k, Ks, rows, stream)
         else:
-            ws = _gemm_workspace(device, need)
-            rc = getattr(lib, "bhi_" + name)(member, x_ptr, split_k, Ks, rows, ws.data_ptr(), ws.numel(), _stream(weight.rem))
+            ws = _gemm_workspace(device, stream, need)
+            rc = getattr(lib, "bhi_" + name)(member, x_ptr, split_k, Ks, rows, ws.data_ptr(), ws.numel(), stream)
+        if rc != 0 and ws is not None:
+            # the launch did not happen or was cut short: its counters may not be zero any more
+            lib.bhi_gemm_workspace_reset(ws.data_ptr(), ws.numel(), stream)
     _lib.check(rc, name)
 
 

@@ -41,6 +41,8 @@ extern "C" {
  *   6 dummy bits per lane   7 max fused batch            8 rANS precision bits
  *   9 stream alignment in 32-bit words                   10 tail padding words
  *  11 task target used by bhi_chunks_per_group           12 max steps per task
+ *  13 sizeof(bhi_gemv_member): a binding checks its own struct against it before it
+ *     passes arrays of members (the struct has grown once, by its last field)
  * Returns the number of constants available. */
 int bhi_constants(int32_t* out, int n);
 
@@ -209,6 +211,16 @@ int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch);
 int bhi_gemm_bf16_huffman_static(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
                                  void* stream);
 int64_t bhi_gemm_static_workspace_bytes(void);
+
+/* No counterpart in the reference.  bhi_device_init: looks up, on the current device, what the
+ * library otherwise looks up at the first call that needs it (the address of the built-in
+ * workspace); call it once per device outside any stream capture if the first use of
+ * bhi_gemm_bf16_huffman_static may happen under capture.  bhi_gemm_workspace_reset: enqueues a
+ * kernel that zeroes a workspace of the fused matrix product (not a memset node, so it may be
+ * captured): for a workspace whose last launch failed or was abandoned, whose counters may be
+ * non-zero. */
+int bhi_device_init(void);
+int bhi_gemm_workspace_reset(void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Readers for weights that were compressed by the reference package itself: same tensors
  * as the reference's huffman_decode / ans_decode ops (kernel.cu:534-587, 878-919) IN THE

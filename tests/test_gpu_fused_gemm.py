@@ -68,3 +68,67 @@ def test_more_than_32_rows_still_decode_then_gemm(cuda):
     x = torch.randn(40, 512, generator=torch.Generator().manual_seed(2)).bfloat16().cuda()
     y = torch.nn.functional.linear(x, mod)
     torch.testing.assert_close(y, torch.nn.functional.linear(x, w.cuda()))
+
+
+def test_k_slice_hand_over_survives_hundreds_of_alternating_launches(cuda):
+    """Two K-sliced shapes take turns on ONE workspace, a few hundred launches with no host
+    synchronisation in between: every result must have the bits of the first one (a partial sum
+    read before its store had landed, or a counter left non-zero, would show as a difference)."""
+    torch.manual_seed(3)
+    cases = []
+    for M, K, rows in ((1024, 4096, 16), (512, 6144, 32)):
+        w = gaussian_weight(M, K, seed=M)
+        mod = _cls("huffman").compress(w).cuda()
+        x = torch.randn(rows, K, generator=torch.Generator().manual_seed(rows)).bfloat16().cuda()
+        first = torch.nn.functional.linear(x, mod)
+        torch.testing.assert_close(first.float(), x.float() @ w.cuda().float().T, rtol=RTOL, atol=ATOL)
+        cases.append((mod, x, first))
+    from bf16_huffman_infer_amd import _lib
+    for mod, x, _ in cases:
+        sk, M, Ks = mod.rem.shape
+        assert _lib.load().bhi_gemm_workspace_bytes(sk, M, Ks, x.shape[0]) > 0, "the case must be cut along K"
+    outs = []
+    for i in range(300):
+        mod, x, _ = cases[i % 2]
+        outs.append(torch.nn.functional.linear(x, mod))
+    torch.cuda.synchronize()
+    for i, y in enumerate(outs):
+        assert torch.equal(y.view(torch.int16), cases[i % 2][2].view(torch.int16)), f"launch {i} differs from the first"
+
+
+def test_workspaces_belong_to_one_stream_each(cuda):
+    from bf16_huffman_infer_amd import ops
+    w = gaussian_weight(1024, 4096, seed=9)
+    mod = _cls("huffman").compress(w).cuda()
+    x = torch.randn(16, 4096, generator=torch.Generator().manual_seed(1)).bfloat16().cuda()
+    want = torch.nn.functional.linear(x, mod)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = torch.nn.functional.linear(x, mod)
+    side.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    here = ops._workspaces[(x.device, torch.cuda.current_stream().cuda_stream)][-1]
+    there = ops._workspaces[(x.device, side.cuda_stream)][-1]
+    assert here.data_ptr() != there.data_ptr()
+
+
+def test_capture_without_a_workspace_takes_the_built_in_one(cuda):
+    """A 16-row product recorded on a stream that has no workspace yet (the capture stream is a
+    new one): the built-in array serves, and every replay gives the eager bits."""
+    w = gaussian_weight(1024, 4096, seed=11)
+    mod = _cls("huffman").compress(w).cuda()
+    x = torch.randn(16, 4096, generator=torch.Generator().manual_seed(4)).bfloat16().cuda()
+    eager = torch.nn.functional.linear(x, mod)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = torch.nn.functional.linear(x, mod)
+    for i in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {i}"
+        x2 = torch.nn.functional.linear(x, mod)                     # eager work of the program between replays
+        assert torch.equal(x2.view(torch.int16), eager.view(torch.int16))

@@ -76,6 +76,34 @@ def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
         _lib.constants()
 
 
+def test_gemm_workspace_is_keyed_by_device_and_stream():
+    """Two streams must get two workspaces (launches on them may overlap); one stream keeps its
+    own, which grows by replacement while the old one stays alive for launches still enqueued."""
+    from bf16_huffman_infer_amd import ops
+    cpu = torch.device("cpu")
+    make = lambda n: torch.zeros(n, dtype=torch.uint8)
+    saved = dict(ops._workspaces)
+    ops._workspaces.clear()
+    try:
+        a = ops._gemm_workspace(cpu, 11, 100, allocate=make)
+        b = ops._gemm_workspace(cpu, 22, 100, allocate=make)
+        assert a.data_ptr() != b.data_ptr()
+        assert ops._gemm_workspace(cpu, 11, 50, allocate=make) is a
+        big = ops._gemm_workspace(cpu, 11, 4 << 20, allocate=make)
+        assert big is not a and big.numel() >= 4 << 20 and not bool(big.any())
+        assert any(t is a for t in ops._workspaces[(cpu, 11)]), "the smaller workspace must stay alive"
+        assert ops._gemm_workspace(cpu, 22, 100, allocate=make) is b
+    finally:
+        ops._workspaces.clear()
+        ops._workspaces.update(saved)
+
+
+def test_binding_checks_the_member_struct_against_the_library():
+    import ctypes
+    from bf16_huffman_infer_amd import _lib
+    assert _lib.constants()["member_bytes"] == ctypes.sizeof(_lib.GemvMember) == 88
+
+
 def test_package_does_not_import_the_oracle():
     import subprocess
     import sys
