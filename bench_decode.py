@@ -274,6 +274,9 @@ def parse_args(argv=None):
     ap.add_argument("--small", action="store_true", help="tiny shapes (smoke run)")
     ap.add_argument("--no-group", action="store_true", help="q/k/v and gate/up as separate launches")
     ap.add_argument("--no-fuse", action="store_true", help="norms, silu*mul and residual additions as separate PyTorch kernels")
+    ap.add_argument("--profile", action="store_true",
+                    help="only the compressed model as it is served (grouped, fused), one run of --tokens tokens, no raw "
+                         "model and no logit comparison: the run to put under rocprofv3 --kernel-trace")
     ap.add_argument("--gold-steps", type=int, default=64,
                     help="teacher-forced steps also run with fp32 matmuls of the raw weights (0: skip)")
     return ap.parse_args(argv)
@@ -296,6 +299,20 @@ def run(args) -> dict:
         runs = [generate(model, prompt, args.tokens) for _ in range(args.repeats)]
         assert all(torch.equal(runs[0][0], r[0]) for r in runs), "generation is not reproducible"
         return runs[0][0], min(r[1] for r in runs)
+
+    if args.profile:
+        from bf16_huffman_infer_amd.cudastream_utils import parallelize_qkv_model
+        convert_all_linear(model, min_out_features=0, progress=False, algo=args.algo)
+        model.to(device)
+        if not args.no_group:
+            parallelize_qkv_model(model)
+            if not args.no_fuse:
+                fuse_neighbours(model)
+        torch.cuda.synchronize()
+        _, secs = generate(model, prompt, args.tokens)
+        return {"workload": "compressed model only (profile run)", "algo": args.algo, "layers": c.layers, "tokens": args.tokens,
+                "prompt": args.prompt, "library_launches_per_token": 4 * c.layers + 1 if not args.no_group else 7 * c.layers + 1,
+                "compressed_tokens_per_s": round(args.tokens / secs, 2), "compressed_ms_per_token": round(secs / args.tokens * 1e3, 4)}
 
     raw_size = get_model_size(model)
     raw_ids, raw_s = best(model)

@@ -652,23 +652,40 @@ def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool 
     return model.load_state_dict(state_dict, strict=strict, assign=True)
 
 
+def prefers_matrix_cores(rows: int, M: int, K: int) -> bool:
+    """Whether ``rows`` <= 8 rows of activations go through the matrix-core kernel rather than the
+    GEMV.  The GEMV re-reads X per wavefront (``rows`` x 256 bytes per step beside 0.7 KB of
+    weights) and spends four dot products per row and step; the matrix-core kernel shares X among
+    the eight wavefronts of a block through LDS and costs the same for 5..8 rows, but starts
+    slower.  Measured on MI355X (us, GEMV / matrix cores): 3584x18944 at 4 rows 26.3 / 25.4, at 8
+    rows 36.0 / 28.7; 12288x4096 at 5 rows 20.5 / 22.6, at 6 rows 24.0 / 22.6, at 8 rows 26.2 / 22.6;
+    4096x12288 at 7 rows 27.0 / 27.5, at 8 rows 28.4 / 27.5; 18944x3584 at 8 rows 30.6 / 30.9; the
+    layers of 4096x4096 and below are 1.3-4 us faster on the GEMV at every row count."""
+    if M % 64 != 0:
+        return False
+    return (rows >= 4 and K >= 16384) or (rows >= 6 and M >= 8192 and K >= 4096) or (rows >= 8 and K >= 12288)
+
+
 def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tensor], fused) -> Tensor:
     assert input.dim() >= 2, input
     shape = input.shape
     input = input.flatten(0, -2)
     if input.size(0) == 0:                       # no rows: nothing to launch
         return input.new_empty((*shape[:-1], weight.rem.shape[1]))
-    if input.size(0) <= MAX_FUSED_BATCH:
+    split_k, M, N = weight.rem.shape
+    wide = (input.size(0) <= MAX_FUSED_BATCH and not isinstance(weight, NibbleWeight) and input.dtype == torch.bfloat16
+            and (bias is None or bias.dtype == torch.bfloat16) and prefers_matrix_cores(input.size(0), M, split_k * N))
+    if input.size(0) <= MAX_FUSED_BATCH and not wide:
         if bias is not None and bias.dtype == torch.bfloat16:
             # the grouped entry point adds the bias in the kernel's last store (same bits, one launch less)
             return linear_grouped(input, [weight], [bias])[0].unflatten(0, shape[:-1])
         output = fused(input)
         if bias is not None:
             output += bias[None, :]
-    elif (input.size(0) <= GEMM_MAX_ROWS and not isinstance(weight, NibbleWeight) and input.dtype == torch.bfloat16
-          and (bias is None or bias.dtype == torch.bfloat16)):
-        # 9..32 rows: decode inside the matrix-core kernel, no BF16 weight in memory
-        split_k, M, N = weight.rem.shape
+    elif wide or (input.size(0) <= GEMM_MAX_ROWS and not isinstance(weight, NibbleWeight) and input.dtype == torch.bfloat16
+                  and (bias is None or bias.dtype == torch.bfloat16)):
+        # 9..32 rows (and fewer where the rule above says so): decode inside the matrix-core kernel,
+        # no BF16 weight in memory
         x = input.view(-1, split_k, N)
         _check_weight_call(weight.rem, weight.exp, x)
         output = torch.empty((x.size(0), M), dtype=torch.bfloat16, device=x.device)

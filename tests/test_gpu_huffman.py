@@ -125,10 +125,18 @@ def test_full_size_layers_round_trip(cuda, algo, kind, M, K):
     ratio = sum(b.numel() * b.element_size() for b in mod.buffers()) / (2 * M * K)
     # short tasks (7 steps for 4608x3584) pay the 64-bit rANS state flush per lane
     assert ratio < (0.75 if algo == "huffman" else 0.78), ratio
-    for bs in (1, 2, 4, 8):
+    from bf16_huffman_infer_amd.functional import mv_ans, mv_huffman
+    for bs in range(1, 9):
         x = torch.randn(bs, K, generator=g, device="cuda").bfloat16()
-        y = torch.nn.functional.linear(x, mod)
         ref = x.float() @ w.float().T
+        # what F.linear chooses for this shape and row count (the GEMV, or the matrix-core kernel) ...
+        y = torch.nn.functional.linear(x, mod)
+        torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
+        # ... and the fused GEMV itself at every batch, which is what the reference's op is
+        if algo == "huffman":
+            y = mv_huffman(mod.rem, mod.exp, x, mod.offsets, mod.LUT1, mod.LUT2, mod.LUT3, mod.LUT4, mod.code_lengths)
+        else:
+            y = mv_ans(mod.rem, mod.exp, x, mod.offsets, mod.LUT)
         torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
 
 

@@ -98,6 +98,18 @@ def test_gemm_workspace_is_keyed_by_device_and_stream():
         ops._workspaces.update(saved)
 
 
+def test_dispatch_rule_between_gemv_and_matrix_cores():
+    """The measured rule: small layers and few rows stay on the GEMV; long-K and large layers move to
+    the matrix-core kernel from 4, 6 or 8 rows."""
+    from bf16_huffman_infer_amd.functional import prefers_matrix_cores
+    for M, K in ((4608, 3584), (3584, 3584), (4096, 4096), (1024, 4096), (18944, 3584)):
+        assert not any(prefers_matrix_cores(r, M, K) for r in range(1, 9)), (M, K)
+    assert [r for r in range(1, 9) if prefers_matrix_cores(r, 3584, 18944)] == [4, 5, 6, 7, 8]
+    assert [r for r in range(1, 9) if prefers_matrix_cores(r, 12288, 4096)] == [6, 7, 8]
+    assert [r for r in range(1, 9) if prefers_matrix_cores(r, 4096, 12288)] == [8]
+    assert not prefers_matrix_cores(8, 3584 + 4, 18944)          # the kernel needs whole blocks of 16 row groups
+
+
 def test_binding_checks_the_member_struct_against_the_library():
     import ctypes
     from bf16_huffman_infer_amd import _lib
