@@ -14,8 +14,37 @@ constexpr int kAnsTableWords = 1 << kAnsPrecision;
 constexpr int kAnsHalf = 4;                     // symbols between two looks at the state
 constexpr int kAnsInitRows = 2;                 // rows 0, 1 of a lane: its initial state
 
+// The decode table in LDS: one 8-byte entry per slot, built from the table buffer's words
+// ((sym<<24)|(freq<<12)|rem, the reference's format) when a block starts:
+//   word 0  freq                 -- an operand of the multiply as it stands
+//   word 1  (sym << 23) | rem    -- rem in the low bits; the symbol where the upper half of the
+//                                   word, moved into one half of a pair word, is `sym << 7`
+// Read with one ds_read_b64, this saves the two field extractions per symbol and the shift per
+// pair of the packed form (eight symbols a step: the kernel is bound by instruction issue).
+struct AnsTable {
+    static constexpr int kLdsWords = 2 * kAnsTableWords;
+    static __device__ __forceinline__ uint2 expand(uint32_t w) {
+        return make_uint2((w >> 12) & 0xFFFu, ((w >> 24) << 23) | (w & 0xFFFu));
+    }
+    template <int THREADS>
+    struct Stage {
+        static_assert(THREADS >= kAnsTableWords, "one slot per thread");
+        uint32_t w;
+        __device__ __forceinline__ void issue(const uint32_t* __restrict__ g) {
+            if (THREADS == kAnsTableWords || (int)threadIdx.x < kAnsTableWords) w = g[threadIdx.x];
+        }
+        __device__ __forceinline__ void commit(uint32_t* __restrict__ lds) const {
+            if (THREADS == kAnsTableWords || (int)threadIdx.x < kAnsTableWords) ((uint2*)lds)[threadIdx.x] = expand(w);
+        }
+    };
+    static __device__ __forceinline__ void fill(uint32_t* __restrict__ lds, const uint32_t* __restrict__ g) {
+        for (int i = threadIdx.x; i < kAnsTableWords; i += blockDim.x) ((uint2*)lds)[i] = expand(g[i]);
+    }
+};
+
 struct AnsCodec {
     using Cursor = AnsCursor;
+    using Table = AnsTable;
     static constexpr bool kTransformsX = true;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr int kTableWords = kAnsTableWords;
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__) { return false; }

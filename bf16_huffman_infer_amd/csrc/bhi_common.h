@@ -178,8 +178,12 @@ typedef __attribute__((address_space(3))) uint32_t lds_u32;
 
 // A lane's view of its task block: a bit position in its own column of rows, and the
 // wavefront's LDS ring of staged rows.  The codec cursors below build on it.
-struct RowRing {
-    uint32_t pos;            // bit position of the lane's window (codec specific bias)
+// POS_SHIFT: `pos` counts bits (5: the Huffman cursor, whose windows start at any bit) or whole
+// rows (0: the rANS cursor, which only ever takes whole words -- advancing by one row is then an
+// add with carry-in off the refill test instead of a select and an add).
+template <int POS_SHIFT>
+struct RowRingT {
+    uint32_t pos;            // position of the lane's window, in bits or rows (codec specific bias)
     uint32_t rhi;            // wave-uniform: rows [0, rhi) have been staged
     uint32_t lim;            // wave-uniform: windows starting below this bit are fully staged
     uint32_t nrows;          // wave-uniform: rows of the block worth staging
@@ -195,12 +199,12 @@ struct RowRing {
         lim = 0;
     }
 
-    // This lane's word of row p >> 5; the next two rows follow at +kLanes, +2*kLanes words.
+    // This lane's word of row p >> POS_SHIFT; the next two rows follow at +kLanes, +2*kLanes words.
     __device__ __forceinline__ const lds_u32* slot_of(uint32_t p) const {
         // v_bfe_u32 + v_lshl_add_u32; written as shift and mask the compiler makes it three
         // instructions on the critical path of every step
         uint32_t slot;
-        asm("v_bfe_u32 %0, %1, 5, %2" : "=v"(slot) : "v"(p), "n"(kRingRowsLog2));
+        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(slot) : "v"(p), "n"(POS_SHIFT), "n"(kRingRowsLog2));
         return ring + slot * kLanes;
     }
 
@@ -225,7 +229,7 @@ struct RowRing {
 
     // windows read rows m..m+2; once the whole block is staged nothing can be missing
     __device__ __forceinline__ void set_lim() {
-        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi - 2) << 5;
+        lim = rhi >= nrows ? 0xFFFFFFFFu : (rhi - 2) << POS_SHIFT;
     }
 
     // Can the next R rows be staged now?  Row r may replace row r - kRingRows once
@@ -240,7 +244,7 @@ struct RowRing {
     template <int R>
     __device__ __forceinline__ bool room_at(uint32_t first) const {
         const uint32_t top = first + R;
-        const uint32_t oldest = top > (uint32_t)kRingRows ? (top - kRingRows) << 5 : 0u;
+        const uint32_t oldest = top > (uint32_t)kRingRows ? (top - kRingRows) << POS_SHIFT : 0u;
         return first < nrows && ballot(pos < oldest) == 0;
     }
 
@@ -269,7 +273,7 @@ struct RowRing {
         set_lim();
     }
 
-    // The lane's window: rows m, m+1, m+2 with m = pos >> 5.
+    // The lane's window: rows m, m+1, m+2 with m = pos >> POS_SHIFT.
     __device__ __forceinline__ void window(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
         // the ring is read unconditionally (a slot address is always valid); lanes whose
         // window is not staged there get it from global memory instead
@@ -285,7 +289,7 @@ struct RowRing {
     // address is kept in range for the others (the stream ends in a zero pad anyway).
     __device__ __forceinline__ void fetch_behind(uint32_t& lo, uint32_t& hi, uint32_t& nx) const {
         const bool staged = pos < lim;
-        const uint32_t* g = bp + (size_t)(staged ? 0u : pos >> 5) * kLanes;
+        const uint32_t* g = bp + (size_t)(staged ? 0u : pos >> POS_SHIFT) * kLanes;
         const uint32_t g0 = g[0], g1 = g[kLanes], g2 = g[2 * kLanes];
         // vmcnt(0) here, inside the rare branch: otherwise the wait lands behind the join
         // and every step would drain the operand loads that are in flight for later steps
@@ -303,6 +307,8 @@ __device__ __forceinline__ uint32_t table_entry(const char* tb, uint32_t w) {
 
 // Per-lane Huffman bit cursor.  pos = bit position - 2: the window is kept shifted left
 // by two so that `window & kTableMask` is the byte address of the table entry.
+typedef RowRingT<5> RowRing;
+
 struct HuffCursor : RowRing {
     uint32_t eptr;           // wave-uniform: escape entries consumed so far
     const uint32_t* ep;      // one past the task block (escape list grows down from here)
@@ -359,8 +365,8 @@ struct HuffCursor : RowRing {
 
 // Per-lane rANS cursor: one 64-bit state, precision 8, table words (sym<<24)|(freq<<12)|rem.
 // The state is looked at after every four symbols; when it has dropped below 2**32 the
-// lane's next row word is shifted in.  pos = 32 * (index of the lane's next row).
-struct AnsCursor : RowRing {
+// lane's next row word is shifted in.  pos = index of the lane's next row.
+struct AnsCursor : RowRingT<0> {
     uint32_t xl, xh;         // the state
 
     __device__ __forceinline__ void open(const uint32_t* __restrict__ words, TaskSpan span, int lane, uint32_t* ring_) {
@@ -371,39 +377,40 @@ struct AnsCursor : RowRing {
     __device__ __forceinline__ void start(const uint32_t*) {
         xl = ring[0];
         xh = ring[kLanes];
-        pos = 2 * 32;
+        pos = 2;
     }
 
-    // one symbol: returns the table word, advances the state
+    // one symbol: returns the second word of its table entry ((sym << 23) | rem), advances the state
     __device__ __forceinline__ uint32_t symbol(const uint32_t* __restrict__ table) {
-        // byte 0 of the state, times four, in one instruction (written as a mask and a shift
+        // byte 0 of the state, times eight, in one instruction (written as a mask and a shift
         // the compiler makes it two; eight symbols per step, the kernel is bound by VALU issue)
         uint32_t off;
         asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
-            : "=v"(off) : "v"(2u), "v"(xl));
-        const uint32_t ent = *(const uint32_t*)((const char*)table + off);
-        const uint32_t f = (ent >> 12) & 0xFFFu;
-        const uint32_t yl = __builtin_amdgcn_alignbit(xh, xl, 8);
-        const uint32_t yh = xh >> 8;
-        const uint64_t lowp = (uint64_t)f * yl + (ent & 0xFFFu);      // v_mad_u64_u32
+            : "=v"(off) : "v"(3u), "v"(xl));
+        const uint2 ent = *(const uint2*)((const char*)table + off);       // {freq, (sym << 23) | rem}
+        // state >> 8 in one instruction (the compiler splits a 64-bit shift by a constant into two)
+        uint64_t y;
+        asm("v_lshrrev_b64 %0, 8, %1" : "=v"(y) : "v"(((uint64_t)xh << 32) | xl));
+        const uint64_t lowp = (uint64_t)ent.x * (uint32_t)y + (ent.y & 0xFFFu);   // v_mad_u64_u32
         xl = (uint32_t)lowp;
-        xh = (uint32_t)(lowp >> 32) + f * yh;                         // f * yh < 2**33 only if the state is valid: < 2**32
-        return ent;
+        // freq <= 256 and y >> 32 < 2**24: a 24-bit multiply-add (the state is valid: < 2**64)
+        xh = __umul24(ent.x, (uint32_t)(y >> 32)) + (uint32_t)(lowp >> 32);
+        return ent.y;
     }
 
     __device__ __forceinline__ void refill(uint32_t word) {
         const bool need = xh == 0u;
         xh = need ? xl : xh;
         xl = need ? word : xl;
-        pos += need ? 32u : 0u;
+        pos += need ? 1u : 0u;
     }
 
-    // two symbols -> one pair entry in the Huffman table's format (a<<7 | b<<23)
+    // two symbols -> one pair entry in the Huffman table's format (a<<7 | b<<23): the upper
+    // halves of the two entry words side by side
     __device__ __forceinline__ uint32_t pair(const uint32_t* __restrict__ table) {
         const uint32_t a = symbol(table);
         const uint32_t b = symbol(table);
-        // the two symbols (byte 3 of the table words) to bytes 0 and 2, then to bits 7 and 23
-        return __builtin_amdgcn_perm(b, a, 0x0C070C03u) << 7;
+        return __builtin_amdgcn_perm(b, a, 0x07060302u);
     }
 
     template <bool UNUSED>

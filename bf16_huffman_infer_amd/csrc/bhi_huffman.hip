@@ -14,6 +14,7 @@ struct HuffCodec {
     using Cursor = HuffCursor;
     static constexpr bool kTransformsX = true;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr int kTableWords = kTableEntries;
+    using Table = PlainTable<kTableEntries>;
     // escaped pairs need the slower walk; the header says whether the matrix has any
     static __device__ __forceinline__ bool variant(const uint8_t* __restrict__ header) { return header_has_esc(header); }
     static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__ header) { return header_flag_word(header); }

@@ -112,7 +112,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     constexpr int kPieces = S * Q * 4 * 16;                   // 16-byte pieces of a window: (step, batch row, 8 columns)
     constexpr int kLoads = (kPieces + kThreads - 1) / kThreads;
     __shared__ uint32_t rings[NW][kRingWords];
-    __shared__ uint32_t lut[Codec::kTableWords];
+    __shared__ uint32_t lut[Codec::Table::kLdsWords];
     __shared__ uint4 xbuf[2][kWindow];
     __shared__ uint32_t is_last;
 
@@ -180,7 +180,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
             if (kc == kc0) {
                 // the table and the first window of X travel with the task's first loads
                 x_load(id.k, id.t0, id.t1);
-                load_table<Codec::kTableWords>(lut, a.table);
+                Codec::Table::fill(lut, a.table);
                 x_store(0);
                 __syncthreads();
             }

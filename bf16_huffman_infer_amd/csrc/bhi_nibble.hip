@@ -16,6 +16,7 @@ struct NibbleCodec {
     using Cursor = NibbleCursor;
     static constexpr bool kTransformsX = false;    // kernels with RMSNorm / SiLU*mul in front of the product are built
     static constexpr int kTableWords = 4;          // base and flags, one 16-byte copy
+    using Table = PlainTable<4>;
     static __device__ __forceinline__ uint32_t variant_word(const uint8_t* __restrict__ lut) {
         return constant_word((const uint32_t*)lut + 1);
     }

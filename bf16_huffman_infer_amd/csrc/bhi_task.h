@@ -42,6 +42,14 @@ struct TableCopy {
     }
 };
 
+// A codec's decode table as LDS holds it.  The plain case: the words of the table buffer, as they are.
+template <int WORDS>
+struct PlainTable {
+    static constexpr int kLdsWords = WORDS;
+    template <int THREADS> using Stage = TableCopy<WORDS, THREADS>;
+    static __device__ __forceinline__ void fill(uint32_t* __restrict__ lds, const uint32_t* __restrict__ g) { load_table<WORDS>(lds, g); }
+};
+
 struct Shape {
     int M, Ks, split_k, nc, steps;      // steps per (split, group)
     uint32_t total_words;
@@ -462,10 +470,10 @@ void decode_kernel(const uint8_t* __restrict__ A_rem, const uint32_t* __restrict
                            uint16_t* __restrict__ Y, const uint32_t* __restrict__ offsets,
                            const uint32_t* __restrict__ table, const uint8_t* __restrict__ header, Shape s) {
     __shared__ uint32_t rings[NW][kRingWords];
-    __shared__ uint32_t lut[Codec::kTableWords];
+    __shared__ uint32_t lut[Codec::Table::kLdsWords];
     // The table's loads go out first and its LDS writes follow the task's own first loads; a
     // wavefront without a task still copies its share and joins the barrier.
-    TableCopy<Codec::kTableWords, NW * kLanes> table_copy;
+    typename Codec::Table::template Stage<NW * kLanes> table_copy;
     table_copy.issue(table);
     auto stage_table = [&]() {
         table_copy.commit(lut);
@@ -544,7 +552,7 @@ __global__ __launch_bounds__(NW * kLanes, min_waves(BS))
 void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int first3, const Group grp) {
     // The partial sums reuse the rings once every task of the block is done.
     __shared__ uint32_t rings[NW][kRingWords];
-    __shared__ uint32_t lut[Codec::kTableWords];
+    __shared__ uint32_t lut[Codec::Table::kLdsWords];
     __shared__ float rms_part[XM == kXRms ? NW * BS : 1];
     // first1..3: first block of members 1..3 (INT_MAX when absent).  Leading scalar arguments
     // are in registers when the wavefront starts (the library is built with kernel-argument
@@ -577,12 +585,12 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
     // (the RMSNorm variant needs its registers for the sums of squares at that point and
     // copies the table in one go instead)
     constexpr bool kEarlyTable = XM != kXRms;
-    TableCopy<Codec::kTableWords, NW * kLanes> table_copy;
+    typename Codec::Table::template Stage<NW * kLanes> table_copy;
     if (kEarlyTable) table_copy.issue(table);
     auto stage_table = [&]() {
         if (!staged) {
             if (kEarlyTable) table_copy.commit(lut);
-            else load_table<Codec::kTableWords>(lut, table);
+            else Codec::Table::fill(lut, table);
             lds_barrier();
             staged = true;
         }
