@@ -426,7 +426,7 @@ def _gemm_workspace(device: torch.device, stream: int, nbytes: int, allocate=Non
     return held[-1]
 
 
-def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
+def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None, static_workspace: bool = False) -> None:
     """``Y = X @ W.T (+ bias)`` for up to 32 rows of ``X`` with ``W`` held compressed
     (:class:`HuffmanWeight` or :class:`ANSWeight`), decoded inside the matrix-core kernel.
 
@@ -434,11 +434,11 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
     rows (``functional.py:405-407, 460-462``).  ``X`` bf16 ``[rows, split_k, Ks]``, ``Y`` bf16
     ``[rows, M]`` written.  Plain function: only enqueues on the current stream.  Products that
     are cut along K keep their partial sums in a workspace that belongs to the (device, stream)
-    pair of the call, allocated at the first such call.  Under stream capture nothing may be
-    allocated: a call that finds no workspace for the capturing stream goes, for a Huffman
-    weight, through the entry point that uses the array built into the library -- ONE array per
-    GPU, shared by every graph captured that way, so replays of two such graphs that overlap on
-    the GPU race; call once on the stream outside the capture to give it a workspace of its own."""
+    pair of the call and is allocated (and zeroed by a fill kernel) at the first such call on
+    that stream -- also under stream capture, where the allocation comes from the graph's own
+    pool and the fill becomes a node in front of the product.  ``static_workspace=True`` (Huffman
+    weights) allocates nothing and uses the array built into the library instead: ONE array per
+    GPU, so launches that take it and may overlap on the GPU (different streams) race."""
     lib = _lib.load()
     split_k, M, Ks = _weight_dims(weight.rem, weight.offsets)
     if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
@@ -456,15 +456,14 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None) -> None:
         need = int(lib.bhi_gemm_workspace_bytes(split_k, M, Ks, rows))
         if need < 0:
             _lib.check(need, name)
-        held = _workspaces.get((device, stream))
         ws = None
         if need == 0:
             rc = getattr(lib, "bhi_" + name)(member, x_ptr, split_k, Ks, rows, None, 0, stream)
-        elif (held is None or held[-1].numel() < need) and torch.cuda.is_current_stream_capturing():
-            # nothing may be allocated under capture: the library's built-in workspace serves
-            if not huffman or need > int(lib.bhi_gemm_static_workspace_bytes()) or device not in _ready_devices:
-                raise RuntimeError("gemm_bf16: no workspace for this stream yet and the stream is capturing; "
-                                   "call once on this stream outside the capture first")
+        elif static_workspace:
+            if not huffman:
+                raise RuntimeError("gemm_bf16: the built-in workspace serves Huffman weights only")
+            if device not in _ready_devices:
+                raise RuntimeError("gemm_bf16: the library has not been used on this device outside a stream capture yet")
             rc = lib.bhi_gemm_bf16_huffman_static(member, x_ptr, split_k, Ks, rows, stream)
         else:
             ws = _gemm_workspace(device, stream, need)

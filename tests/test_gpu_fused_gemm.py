@@ -113,11 +113,13 @@ def test_workspaces_belong_to_one_stream_each(cuda):
     assert here.data_ptr() != there.data_ptr()
 
 
-def test_capture_without_a_workspace_takes_the_built_in_one(cuda):
-    """A 16-row product recorded on a stream that has no workspace yet (the capture stream is a
-    new one): the built-in array serves, and every replay gives the eager bits."""
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+def test_capture_on_a_stream_without_a_workspace(cuda, algo):
+    """A 16-row product recorded on a stream that has no workspace yet (torch captures on a stream of
+    its own): the workspace is allocated from the graph's pool, its fill is a node of the graph, and
+    every replay gives the eager bits -- with the program's own eager work between the replays."""
     w = gaussian_weight(1024, 4096, seed=11)
-    mod = _cls("huffman").compress(w).cuda()
+    mod = _cls(algo).compress(w).cuda()
     x = torch.randn(16, 4096, generator=torch.Generator().manual_seed(4)).bfloat16().cuda()
     eager = torch.nn.functional.linear(x, mod)
     torch.cuda.synchronize()
@@ -130,5 +132,28 @@ def test_capture_without_a_workspace_takes_the_built_in_one(cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {i}"
-        x2 = torch.nn.functional.linear(x, mod)                     # eager work of the program between replays
-        assert torch.equal(x2.view(torch.int16), eager.view(torch.int16))
+        again = torch.nn.functional.linear(x, mod)
+        assert torch.equal(again.view(torch.int16), eager.view(torch.int16))
+
+
+def test_built_in_workspace_on_request(cuda):
+    """``static_workspace=True``: nothing is allocated, eagerly or under capture, and the bits are the same."""
+    from bf16_huffman_infer_amd import ops
+    w = gaussian_weight(1024, 4096, seed=12)
+    mod = _cls("huffman").compress(w).cuda()
+    x = torch.randn(16, 1, 4096, generator=torch.Generator().manual_seed(5)).bfloat16().cuda()
+    want = torch.nn.functional.linear(x.view(16, 4096), mod)
+    got = torch.empty_like(want)
+    ops.gemm_bf16(mod, x, got, static_workspace=True)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    graph = torch.cuda.CUDAGraph()
+    rec = torch.empty_like(want)
+    with torch.cuda.graph(graph):
+        ops.gemm_bf16(mod, x, rec, static_workspace=True)
+    for i in range(2):
+        rec.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(rec.view(torch.int16), want.view(torch.int16)), f"replay {i}"
+    with pytest.raises(RuntimeError, match="Huffman"):
+        ops.gemm_bf16(_cls("ans").compress(w).cuda(), x, got, static_workspace=True)
