@@ -47,10 +47,12 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 #define BHI_MMA_LAST_ACQUIRES 1
 #endif
 constexpr int kMmaSeg = 4;                   // steps per window
-// wavefronts (row groups) per block: LDS holds two windows of X (8 KB per batch quad) beside
-// the table and the rings; up to 16 rows two 8-wavefront blocks fit a compute unit, above
-// that one block of 16
-constexpr int mma_waves(int Q) { return Q <= 4 ? 8 : 16; }
+// Wavefronts (row groups) per block.  LDS holds two windows of X (8 KB per batch quad) beside
+// the table and the rings: up to 16 rows two 8-wavefront blocks fit a compute unit, and one
+// block of 12 or of 16 at any batch.  Which one a launch takes is a matter of how evenly its
+// blocks cover the 256 compute units (mma_plan below).
+constexpr int kMmaWavesSmall = 8, kMmaWavesMid = 12, kMmaWavesLarge = 16;
+constexpr int kMmaSmallUpToQ = 4;            // 8-wavefront blocks: batch quads 1..4
 constexpr int kMmaMaxBatch = 32;
 constexpr int kMmaMaxSlices = 8;
 constexpr int kMmaSliceBelowGroups = 2048;   // weights with fewer row groups are cut along K
@@ -104,7 +106,7 @@ __host__ __device__ inline long long mma_partial_floats(int M, int batch, int sl
 }
 
 template <class Codec, int Q, int NW>
-__global__ __launch_bounds__(NW * kLanes, 4)
+__global__ __launch_bounds__(NW * kLanes, (NW == kMmaWavesMid ? 3 : 4))     // wavefronts per SIMD that the blocks of a compute unit add up to
 void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     constexpr int S = kMmaSeg;
     constexpr int kWindow = S * Q * kLanes;                   // 16-byte units of one X window
@@ -120,7 +122,11 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     const int lane = threadIdx.x & (kLanes - 1);
     const int wave = (int)uniform(threadIdx.x / kLanes);
     const int rb = (int)blockIdx.x / a.slices, ks = (int)blockIdx.x % a.slices;
-    const int g = rb * NW + wave;
+    // a block past the last row group (M / 4 need not be a multiple of NW) repeats that group
+    // without storing anything: its wavefronts still load their share of X and meet the barriers
+    const int G = s.M / kGroupRows;
+    const bool real = rb * NW + wave < G;
+    const int g = real ? rb * NW + wave : G - 1;
     const int per_group = s.split_k * s.nc;
     const int tpk = per_group / a.slices;
     const int kc0 = ks * tpk, kc1 = kc0 + tpk;
@@ -134,8 +140,8 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
 
     // ---- X staging: piece p of a window = (step i, batch row r = 4q + j, column group b); the
     // thread that loads it writes it where lane 4b + j will read it
-    static_assert(kLoads <= 2, "two pieces per thread at most");
-    uint4 xg0 = make_uint4(0, 0, 0, 0), xg1 = make_uint4(0, 0, 0, 0);     // (named registers: an array would live in scratch memory)
+    static_assert(kLoads <= 3, "three pieces per thread at most");
+    uint4 xg0 = make_uint4(0, 0, 0, 0), xg1 = make_uint4(0, 0, 0, 0), xg2 = make_uint4(0, 0, 0, 0);     // (named registers: an array would live in scratch memory)
     auto piece_load = [&](uint4& dst, int n, int k, int t0, int t_end) __attribute__((always_inline)) {
         const int p = (int)threadIdx.x + n * kThreads;
         if (kPieces % kThreads == 0 || p < kPieces) {
@@ -156,10 +162,12 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     auto x_load = [&](int k, int t0, int t_end) __attribute__((always_inline)) {       // window starting at step t0 of split k; the task ends at t_end
         piece_load(xg0, 0, k, t0, t_end);
         if (kLoads > 1) piece_load(xg1, 1, k, t0, t_end);
+        if (kLoads > 2) piece_load(xg2, 2, k, t0, t_end);
     };
     auto x_store = [&](int par) __attribute__((always_inline)) {
         piece_store(xg0, 0, par);
         if (kLoads > 1) piece_store(xg1, 1, par);
+        if (kLoads > 2) piece_store(xg2, 2, par);
     };
 
     typename Codec::Cursor cur;
@@ -226,7 +234,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
         }
     }
     if (a.slices == 1) {
-        if (lane < 4) {
+        if (real && lane < 4) {
 #pragma unroll
             for (int q = 0; q < Q; ++q) {
                 const int batch = 4 * q + lane;
@@ -251,7 +259,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     // the acquire in the last block: +0.1-0.4 us).  A cache-wide fence per WAVEFRONT, 6144 of
     // them, made the launch take 270 us.  What this relies on beyond the language's memory model:
     // an acknowledged agent-scope store is visible to agent-scope loads of every die.
-    if (lane < 4) {
+    if (real && lane < 4) {
 #pragma unroll
         for (int q = 0; q < Q; ++q) {
             const int batch = 4 * q + lane;
@@ -277,6 +285,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     const int rows_here = kGroupRows * NW;
     for (int e = threadIdx.x; e < B * rows_here; e += kThreads) {
         const int batch = e / rows_here, row = rb * rows_here + e % rows_here;
+        if (row >= s.M) continue;
         float v = 0.f;
         for (int k = 0; k < a.slices; ++k)
             v += __hip_atomic_load(a.partial + ((size_t)k * B + batch) * s.M + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -287,48 +296,84 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
 
 }  // namespace bhi
 
-// K slices of a launch: the divisor d of the tasks per row group that minimises a small cost
-// model, in units of steps.  A block walks (tasks per group / d) tasks and pays about six
-// steps' worth of start; with at most one block per compute unit (256) the blocks run at
-// full pace, with two 8-wavefront blocks on a unit at two thirds of it, and blocks beyond
-// what is resident at once (512 of 8 wavefronts, 256 of 16) wait for a whole round; every
-// slice adds a round trip of partial sums (two steps' worth).  The model reproduces the order
-// measured at 16 / 32 rows: 4096x12288 (6 tasks of 16 steps) 2 slices 32 us, 3 slices 33 us,
-// 6 slices 41 us, none 50 us / 3 slices 44 us, 2 slices 55 us, 6 slices 59 us;
-// 3584x18944 (4 tasks of 37 steps) 4 slices 36 us, 2 slices 42 us; 4096x4096 (4 tasks of 8
-// steps) 2 slices 17 us, 4 slices 20 us; 4608x3584 2 slices 20 / 29 us, 4 slices 24 / 42 us.
-static inline int mma_slices(const bhi::Shape& s, int nw) {
+// Shape of a launch: wavefronts per block and K slices, by a small cost model in units of steps.
+//
+// A block of NW wavefronts covers NW row groups and walks (tasks per group / d) tasks when the
+// row group's tasks are dealt to d blocks (K slices, d a divisor); it pays about six steps'
+// worth of start, and every slice adds a round trip of partial sums (two steps' worth).  The
+// pace of a block depends on how many wavefronts share its compute unit: measured on
+// 4096-column weights at 16 rows, a unit with 8 / 12 / 16 resident wavefronts gets through
+// 1 / 1.26 / 1.51 row groups in the time a lone 8-wavefront block needs for one (8192 rows,
+// 256 blocks: 21.1 us; 12288 rows as 256 blocks of 12: 25.0 us; 16384 rows, 512 blocks of 8:
+// 27.9 us).  What the model is there to avoid is a grid that covers the 256 units unevenly:
+// 12288 rows as 384 blocks of 8 put two blocks on half of the units and one on the rest and
+// take as long as 16384 rows (27.7 us; at 32 rows 192 blocks of 16 leave a quarter of the
+// units idle: 37.2 us against 32.2 us for 256 blocks of 12).  Blocks beyond what is resident
+// at once (512 of 8 wavefronts up to 16 rows, else 256) wait for a round; a last round of at
+// most 256 blocks of 8 runs at the lone block's pace (18944x3584 at 16 rows, 592 blocks of 8:
+// 38.1 us, 395 blocks of 12: 39.5 us).  The 8-wavefront block (16 above 16 rows) stays unless
+// another shape is at least 4 % cheaper, and so does a smaller number of slices: the model is
+// no more exact than that.
+// The model reproduces the order measured at 16 / 32 rows for the slices as well: 4096x12288
+// (6 tasks of 16 steps) 2 slices 32 us, 3 slices 33 us, 6 slices 41 us, none 50 us / 3 slices
+// 44 us, 2 slices 55 us, 6 slices 59 us; 3584x18944 (4 tasks of 37 steps) 4 slices 36 us,
+// 2 slices 42 us; 4096x4096 (4 tasks of 8 steps) 2 slices 17 us, 4 slices 20 us.
+struct MmaPlan { int nw, slices; };
+
+static inline MmaPlan mma_plan(const bhi::Shape& s, int Q) {
     using namespace bhi;
     const int G = s.M / kGroupRows, per_group = s.split_k * s.nc;
-    if (G >= kMmaSliceBelowGroups) return 1;
-    const long long row_blocks = G / nw;
     const double task_steps = (double)s.steps / s.nc;
-    int best = 1;
+    const int max_slices = G >= kMmaSliceBelowGroups ? 1 : kMmaMaxSlices;
+    MmaPlan best = {0, 1};
     double best_cost = 0;
-    for (int d = 1; d <= kMmaMaxSlices && d <= per_group; ++d) {
-        if (per_group % d != 0) continue;
-        const long long blocks = row_blocks * d;
-        double pace;
-        if (nw <= 8) pace = blocks <= 256 ? 1.0 : 1.5 * (double)((blocks + 511) / 512);
-        else pace = (double)((blocks + 255) / 256);
-        const double cost = pace * (per_group / d * task_steps + 6.0) + 2.0 * d;
-        if (d == 1 || cost < best_cost) { best = d; best_cost = cost; }
+    const bool small = Q <= kMmaSmallUpToQ;
+    const int candidates[3] = {small ? kMmaWavesSmall : kMmaWavesLarge, kMmaWavesMid, small ? kMmaWavesLarge : 0};
+    for (int nw : candidates) {
+        if (nw == 0) continue;
+        const long long row_blocks = (G + nw - 1) / nw;
+        MmaPlan here = {nw, 1};
+        double here_cost = 0;
+        for (int d = 1; d <= max_slices && d <= per_group; ++d) {
+            if (per_group % d != 0) continue;
+            const long long blocks = row_blocks * d;
+            double pace;
+            if (nw == kMmaWavesSmall) {
+                const long long rest = blocks % 512;
+                pace = 1.325 * (double)(blocks / 512) + (rest == 0 ? 0.0 : (rest <= 256 ? 1.0 : 1.325));
+            } else {
+                pace = (nw == kMmaWavesMid ? 1.19 : 1.325) * (double)((blocks + 255) / 256);
+            }
+            const double cost = pace * (per_group / d * task_steps + 6.0) + 2.0 * d;
+            if (d == 1 || cost < 0.96 * here_cost) { here = MmaPlan{nw, d}; here_cost = cost; }
+        }
+        if (best.nw == 0 || here_cost < 0.96 * best_cost) { best = here; best_cost = here_cost; }
     }
     return best;
 }
 
 static inline int64_t mma_workspace_bytes(const bhi::Shape& s, int batch) {
     using namespace bhi;
-    const int slices = mma_slices(s, mma_waves((batch + 3) / 4));
+    const int slices = mma_plan(s, (batch + 3) / 4).slices;
     return slices > 1 ? kMmaCounterBytes + mma_partial_floats(s.M, batch, slices) * 4 : 0;
 }
 
-template <class Codec, int Q>
-static inline void launch_mma_q(const bhi::MmaArgs& a, const uint16_t* x, hipStream_t stream) {
+template <class Codec, int Q, int NW>
+static inline void launch_mma_qn(const bhi::MmaArgs& a, const uint16_t* x, hipStream_t stream) {
     using namespace bhi;
-    constexpr int NW = mma_waves(Q);
-    const dim3 grid((unsigned)(a.s.M / (kGroupRows * NW) * a.slices)), block(NW * kLanes);
+    const int G = a.s.M / kGroupRows;
+    const dim3 grid((unsigned)((G + NW - 1) / NW * a.slices)), block(NW * kLanes);
     hipLaunchKernelGGL((mma_kernel<Codec, Q, NW>), grid, block, 0, stream, x, a);
+}
+
+template <class Codec, int Q>
+static inline void launch_mma_q(const bhi::MmaArgs& a, int nw, const uint16_t* x, hipStream_t stream) {
+    using namespace bhi;
+    if constexpr (Q <= kMmaSmallUpToQ) {
+        if (nw == kMmaWavesSmall) return launch_mma_qn<Codec, Q, kMmaWavesSmall>(a, x, stream);
+    }
+    if (nw == kMmaWavesMid) return launch_mma_qn<Codec, Q, kMmaWavesMid>(a, x, stream);
+    launch_mma_qn<Codec, Q, kMmaWavesLarge>(a, x, stream);
 }
 
 template <class Codec>
@@ -343,9 +388,9 @@ static inline int launch_mma(const bhi_gemv_member& m, const void* X, int split_
         return bhi_fail(BHI_ELAYOUT, "decode table has the wrong size");
     Shape s;
     if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &s)) return rc;
-    const int Q = (batch + 3) / 4, nw = mma_waves(Q);
-    if (m.M % (kGroupRows * nw) != 0) return bhi_fail(BHI_EINVAL, "M must be a multiple of 64");
-    const int slices = mma_slices(s, nw);
+    const int Q = (batch + 3) / 4;
+    const MmaPlan plan = mma_plan(s, Q);
+    const int slices = plan.slices;
     const int64_t need = mma_workspace_bytes(s, batch);
     if (slices > 1 && (!workspace || workspace_bytes < need)) return bhi_fail(BHI_EINVAL, "workspace too small: see bhi_gemm_workspace_bytes");
     MmaArgs a;
@@ -357,14 +402,14 @@ static inline int launch_mma(const bhi_gemv_member& m, const void* X, int split_
     a.partial = (float*)((char*)workspace + kMmaCounterBytes);
     const uint16_t* x = (const uint16_t*)X;
     switch (Q) {
-        case 1: launch_mma_q<Codec, 1>(a, x, stream); break;
-        case 2: launch_mma_q<Codec, 2>(a, x, stream); break;
-        case 3: launch_mma_q<Codec, 3>(a, x, stream); break;
-        case 4: launch_mma_q<Codec, 4>(a, x, stream); break;
-        case 5: launch_mma_q<Codec, 5>(a, x, stream); break;
-        case 6: launch_mma_q<Codec, 6>(a, x, stream); break;
-        case 7: launch_mma_q<Codec, 7>(a, x, stream); break;
-        default: launch_mma_q<Codec, 8>(a, x, stream); break;
+        case 1: launch_mma_q<Codec, 1>(a, plan.nw, x, stream); break;
+        case 2: launch_mma_q<Codec, 2>(a, plan.nw, x, stream); break;
+        case 3: launch_mma_q<Codec, 3>(a, plan.nw, x, stream); break;
+        case 4: launch_mma_q<Codec, 4>(a, plan.nw, x, stream); break;
+        case 5: launch_mma_q<Codec, 5>(a, plan.nw, x, stream); break;
+        case 6: launch_mma_q<Codec, 6>(a, plan.nw, x, stream); break;
+        case 7: launch_mma_q<Codec, 7>(a, plan.nw, x, stream); break;
+        default: launch_mma_q<Codec, 8>(a, plan.nw, x, stream); break;
     }
     return 0;
 }

@@ -661,8 +661,6 @@ def prefers_matrix_cores(rows: int, M: int, K: int) -> bool:
     rows 36.0 / 28.7; 12288x4096 at 5 rows 20.5 / 22.6, at 6 rows 24.0 / 22.6, at 8 rows 26.2 / 22.6;
     4096x12288 at 7 rows 27.0 / 27.5, at 8 rows 28.4 / 27.5; 18944x3584 at 8 rows 30.6 / 30.9; the
     layers of 4096x4096 and below are 1.3-4 us faster on the GEMV at every row count."""
-    if M % 64 != 0:
-        return False
     return (rows >= 4 and K >= 16384) or (rows >= 6 and M >= 8192 and K >= 4096) or (rows >= 8 and K >= 12288)
 
 

@@ -62,6 +62,25 @@ def test_full_size_fallback_shapes(cuda, algo, M, K, rows):
     assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
 
 
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("rows", [3, 12, 20, 32])
+@pytest.mark.parametrize("M,K", [(128, 512), (640, 2048), (1408, 1024), (12160, 512), (12416, 512)])
+def test_row_counts_that_fill_no_whole_block(cuda, algo, rows, M, K):
+    """M / 4 row groups that are no multiple of the 12 a block may hold (the last block repeats the
+    last group and stores nothing for the repeats), with and without K slices; 12160 rows at up to
+    16 rows of X and every case above 16 take blocks of 12."""
+    from bf16_huffman_infer_amd import ops
+    w = gaussian_weight(M, K, seed=M + rows)
+    mod = _cls(algo).compress(w).cuda()
+    x = torch.randn(rows, K, generator=torch.Generator().manual_seed(rows)).bfloat16().cuda()
+    y = torch.full((rows, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+    guard = torch.full((4096,), 7.0, dtype=torch.bfloat16, device="cuda")       # allocated right behind y
+    ops.gemm_bf16(mod, x.view(rows, *mod.rem.shape[::2]), y)
+    ref = x.float() @ w.cuda().float().T
+    torch.testing.assert_close(y.float(), ref, rtol=RTOL, atol=ATOL)
+    assert bool((guard == 7.0).all())
+
+
 def test_more_than_32_rows_still_decode_then_gemm(cuda):
     w = gaussian_weight(256, 512, seed=7)
     mod = _cls("huffman").compress(w).cuda()
