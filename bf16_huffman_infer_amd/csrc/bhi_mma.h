@@ -53,6 +53,15 @@ constexpr int kMmaSeg = 4;                   // steps per window
 // blocks cover the 256 compute units (mma_plan below).
 constexpr int kMmaWavesSmall = 8, kMmaWavesMid = 12, kMmaWavesLarge = 16;
 constexpr int kMmaSmallUpToQ = 4;            // 8-wavefront blocks: batch quads 1..4
+// Blocks of NW wavefronts that a compute unit holds at Q batch quads: by LDS (rings 4.5 KB per
+// wavefront, table up to 8 KB, X windows 8 KB per quad, 160 KB per unit) and by registers
+// (65-73 up to two quads: six wavefronts per SIMD; 84-102 up to four quads: four; above: three
+// or four)
+constexpr int mma_resident_blocks(int Q, int NW) {
+    return Q == 1 ? (NW == kMmaWavesSmall ? 3 : (NW == kMmaWavesMid ? 2 : 1))
+         : Q == 2 ? (NW == kMmaWavesLarge ? 1 : 2)
+         : Q <= 4 ? (NW == kMmaWavesSmall ? 2 : 1) : 1;
+}
 constexpr int kMmaMaxBatch = 32;
 constexpr int kMmaMaxSlices = 8;
 constexpr int kMmaSliceBelowGroups = 2048;   // weights with fewer row groups are cut along K
@@ -106,7 +115,7 @@ __host__ __device__ inline long long mma_partial_floats(int M, int batch, int sl
 }
 
 template <class Codec, int Q, int NW>
-__global__ __launch_bounds__(NW * kLanes, (NW == kMmaWavesMid ? 3 : 4))     // wavefronts per SIMD that the blocks of a compute unit add up to
+__global__ __launch_bounds__(NW * kLanes, mma_resident_blocks(Q, NW) * NW / 4)     // wavefronts per SIMD that the blocks of a compute unit add up to
 void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     constexpr int S = kMmaSeg;
     constexpr int kWindow = S * Q * kLanes;                   // 16-byte units of one X window
@@ -305,20 +314,26 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
 // 4096-column weights at 16 rows, a unit with 8 / 12 / 16 resident wavefronts gets through
 // 1 / 1.26 / 1.51 row groups in the time a lone 8-wavefront block needs for one (8192 rows,
 // 256 blocks: 21.1 us; 12288 rows as 256 blocks of 12: 25.0 us; 16384 rows, 512 blocks of 8:
-// 27.9 us).  What the model is there to avoid is a grid that covers the 256 units unevenly:
-// 12288 rows as 384 blocks of 8 put two blocks on half of the units and one on the rest and
-// take as long as 16384 rows (27.7 us; at 32 rows 192 blocks of 16 leave a quarter of the
-// units idle: 37.2 us against 32.2 us for 256 blocks of 12).  Blocks beyond what is resident
-// at once (512 of 8 wavefronts up to 16 rows, else 256) wait for a round; a last round of at
-// most 256 blocks of 8 runs at the lone block's pace (18944x3584 at 16 rows, 592 blocks of 8:
-// 38.1 us, 395 blocks of 12: 39.5 us).  The 8-wavefront block (16 above 16 rows) stays unless
-// another shape is at least 4 % cheaper, and so does a smaller number of slices: the model is
-// no more exact than that.
-// The model reproduces the order measured at 16 / 32 rows for the slices as well: 4096x12288
+// 27.9 us), and 24 do no better than 16 (18944x3584 at 8 rows).  What the model is there to
+// avoid is a grid that covers the 256 units unevenly: 12288 rows as 384 blocks of 8 put two
+// blocks on half of the units and one on the rest and take as long as 16384 rows (27.7 us; at
+// 32 rows 192 blocks of 16 leave a quarter of the units idle: 37.2 us against 32.2 us for 256
+// blocks of 12).  Blocks beyond what is resident at once wait for a round; the last round runs
+// at the pace of the wavefronts it puts on a unit (18944x3584 at 16 rows, 592 blocks of 8:
+// 38.1 us, 395 blocks of 12: 39.5 us; at 8 rows, where two blocks of 12 fit a unit: 31.0 and
+// 26.3 us).  The 8-wavefront block (16 above 16 rows) stays unless another shape is at least
+// 4 % cheaper, and so does a smaller number of slices: the model is no more exact than that.
+// It reproduces the order measured at 16 / 32 rows for the slices as well: 4096x12288
 // (6 tasks of 16 steps) 2 slices 32 us, 3 slices 33 us, 6 slices 41 us, none 50 us / 3 slices
 // 44 us, 2 slices 55 us, 6 slices 59 us; 3584x18944 (4 tasks of 37 steps) 4 slices 36 us,
 // 2 slices 42 us; 4096x4096 (4 tasks of 8 steps) 2 slices 17 us, 4 slices 20 us.
 struct MmaPlan { int nw, slices; };
+
+// time of a row group on a unit that holds `waves` wavefronts, relative to a lone block of 8
+static inline double mma_pace(int waves) {
+    const double through = waves <= 8 ? 1.0 : (waves <= 12 ? 1.26 : 1.51);
+    return waves / 8.0 / through;
+}
 
 static inline MmaPlan mma_plan(const bhi::Shape& s, int Q) {
     using namespace bhi;
@@ -332,18 +347,15 @@ static inline MmaPlan mma_plan(const bhi::Shape& s, int Q) {
     for (int nw : candidates) {
         if (nw == 0) continue;
         const long long row_blocks = (G + nw - 1) / nw;
+        const int resident = mma_resident_blocks(Q, nw);
         MmaPlan here = {nw, 1};
         double here_cost = 0;
         for (int d = 1; d <= max_slices && d <= per_group; ++d) {
             if (per_group % d != 0) continue;
             const long long blocks = row_blocks * d;
-            double pace;
-            if (nw == kMmaWavesSmall) {
-                const long long rest = blocks % 512;
-                pace = 1.325 * (double)(blocks / 512) + (rest == 0 ? 0.0 : (rest <= 256 ? 1.0 : 1.325));
-            } else {
-                pace = (nw == kMmaWavesMid ? 1.19 : 1.325) * (double)((blocks + 255) / 256);
-            }
+            const long long rest = blocks % (256 * resident);
+            double pace = mma_pace(nw * resident) * (double)(blocks / (256 * resident));
+            if (rest > 0) pace += mma_pace(nw * (int)((rest + 255) / 256));
             const double cost = pace * (per_group / d * task_steps + 6.0) + 2.0 * d;
             if (d == 1 || cost < 0.96 * here_cost) { here = MmaPlan{nw, d}; here_cost = cost; }
         }

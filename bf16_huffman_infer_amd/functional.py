@@ -453,7 +453,15 @@ def linear_grouped(input: Tensor, weights, biases=None, *, residuals=None, input
         biases = [None if b is None else b.detach().contiguous() for b in biases]
     if residuals is not None:
         residuals = [None if r is None else r.detach().reshape(x.size(0), -1).contiguous() for r in residuals]
-    gemv_bf16_grouped(weights, x.contiguous(), ys, biases, residuals, mode, aux, float(eps))
+    if (mode == _ops.X_PLAIN and (residuals is None or all(r is None for r in residuals))
+            and not isinstance(first, NibbleWeight)
+            and all(prefers_matrix_cores(x.size(0), w.rem.shape[1], split_k * N) for w in weights)):
+        # layers this large are faster through the matrix-core kernel, one launch per member
+        x = x.contiguous()
+        for i, (w, y) in enumerate(zip(weights, ys)):
+            gemm_bf16(w, x, y, None if biases is None else biases[i])
+    else:
+        gemv_bf16_grouped(weights, x.contiguous(), ys, biases, residuals, mode, aux, float(eps))
     return [y.unflatten(0, shape[:-1]) for y in ys]
 
 
@@ -654,14 +662,33 @@ def load_compressed_state_dict(model: nn.Module, state_dict: dict, strict: bool 
 
 def prefers_matrix_cores(rows: int, M: int, K: int) -> bool:
     """Whether ``rows`` <= 8 rows of activations go through the matrix-core kernel rather than the
-    GEMV.  The GEMV re-reads X per wavefront (``rows`` x 256 bytes per step beside 0.7 KB of
-    weights) and spends four dot products per row and step; the matrix-core kernel shares X among
-    the eight wavefronts of a block through LDS and costs the same for 5..8 rows, but starts
-    slower.  Measured on MI355X (us, GEMV / matrix cores): 3584x18944 at 4 rows 26.3 / 25.4, at 8
-    rows 36.0 / 28.7; 12288x4096 at 5 rows 20.5 / 22.6, at 6 rows 24.0 / 22.6, at 8 rows 26.2 / 22.6;
-    4096x12288 at 7 rows 27.0 / 27.5, at 8 rows 28.4 / 27.5; 18944x3584 at 8 rows 30.6 / 30.9; the
-    layers of 4096x4096 and below are 1.3-4 us faster on the GEMV at every row count."""
-    return (rows >= 4 and K >= 16384) or (rows >= 6 and M >= 8192 and K >= 4096) or (rows >= 8 and K >= 12288)
+    GEMV.  The GEMV spends four dot products per row and step and one load of X per row; the
+    matrix-core kernel shares X among the wavefronts of a block through LDS and costs the same for
+    5..8 rows, but starts slower and keeps fewer wavefronts on a compute unit.  Measured on MI355X
+    (us, GEMV / matrix cores):
+
+    ===========  ===========  ===========  ===========  ===========
+    M x K        4 rows       5 rows       6 rows       8 rows
+    ===========  ===========  ===========  ===========  ===========
+    3584x18944   26.4 / 25.9  29.3 / 28.4  31.5 / 28.7  36.8 / 29.3
+    14336x4096   21.8 / 20.5  23.6 / 22.5  25.2 / 22.5  28.4 / 22.5
+    18944x3584   23.4 / 23.9  25.3 / 26.1  27.0 / 26.1  30.8 / 26.2
+    12288x4096   19.0 / 19.4  20.6 / 21.2  23.9 / 21.2  26.4 / 21.2
+    11008x4096   18.6 / 19.0  20.3 / 20.7  23.2 / 20.8  25.3 / 20.8
+    4096x14336   21.9 / 22.8  24.1 / 24.4  26.0 / 24.8  29.5 / 25.5
+    4096x12288   22.1 / 26.1  24.6 / 27.7  25.7 / 27.8  28.6 / 28.0
+    4096x11008   18.6 / 20.7  20.5 / 22.7  21.7 / 23.1  24.7 / 23.8
+    8192x8192    23.1 / 27.7  25.1 / 30.0  27.1 / 30.2  30.8 / 30.3
+    ===========  ===========  ===========  ===========  ===========
+
+    and the layers of 6144x4096 and below are 0.4-4 us faster on the GEMV at every row count; output
+    layers the size of a vocabulary are faster on the matrix cores from 4 rows (152064x3584:
+    180 / 148, 202 / 184, 225 / 185 us at 4, 6, 8 rows; 37888x3584: 44.4 / 39.8, 52.2 / 48.7, 58.7 / 48.9)."""
+    if rows >= 8 and K >= 11008:
+        return True
+    if rows >= 6 and ((M >= 10240 and K >= 3584) or K >= 14336):
+        return True
+    return rows >= 4 and (K >= 16384 or (M >= 14336 and K >= 4096) or (M >= 32768 and K >= 3584))
 
 
 def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tensor], fused) -> Tensor:

@@ -53,6 +53,31 @@ def test_grouped_equals_single_launches(cuda, algo, bs, K, Ms):
             assert worst <= 0, f"biased member off by {worst} beyond its bound"
 
 
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("bs", [5, 6, 8])
+def test_group_of_layers_that_prefer_the_matrix_cores(cuda, algo, bs):
+    """Two 10240x3584 weights from six rows on: every member goes through the matrix-core kernel
+    (one launch each), with the bits of its own ``F.linear`` call and a bias added in the kernel;
+    at five rows the group stays one GEMV launch."""
+    from bf16_huffman_infer_amd.functional import linear_grouped, prefers_matrix_cores
+    assert prefers_matrix_cores(6, 10240, 3584) and not prefers_matrix_cores(5, 10240, 3584)
+    M, K = 10240, 3584
+    ws = [gaussian_weight(M, K, seed=41).cuda(), student_t_weight(M, K, seed=42).cuda()]
+    mods = [_cls(algo).compress(w).cuda() for w in ws]
+    biases = [None, torch.randn(M, generator=torch.Generator().manual_seed(3)).bfloat16().cuda() * 0.1]
+    x = torch.randn(bs, K, generator=torch.Generator().manual_seed(8)).bfloat16().cuda()
+    outs = [torch.empty(bs, M, dtype=torch.bfloat16, device="cuda") for _ in ws]
+    got = linear_grouped(x, mods, biases, outs=outs)
+    for w, mod, b, y, o in zip(ws, mods, biases, got, outs):
+        assert y.data_ptr() == o.data_ptr()
+        single = torch.nn.functional.linear(x, mod, b)
+        assert torch.equal(y.view(torch.int16), single.view(torch.int16))
+        prod = x.float() @ w.float().T
+        ref = prod if b is None else prod + b.float()
+        bound = ATOL + RTOL * ref.abs() + (0 if b is None else 2.0 ** -8) * prod.abs()
+        assert ((y.float() - ref).abs() - bound).max().item() <= 0
+
+
 @pytest.mark.parametrize("algo", ["huffman", "ans", "nibble"])
 @pytest.mark.parametrize("bs", [1, 5])
 def test_oversubscribed_group_of_long_tasks(cuda, algo, bs):

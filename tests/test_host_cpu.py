@@ -102,12 +102,13 @@ def test_dispatch_rule_between_gemv_and_matrix_cores():
     """The measured rule: small layers and few rows stay on the GEMV; long-K and large layers move to
     the matrix-core kernel from 4, 6 or 8 rows."""
     from bf16_huffman_infer_amd.functional import prefers_matrix_cores
-    for M, K in ((4608, 3584), (3584, 3584), (4096, 4096), (1024, 4096), (18944, 3584)):
+    for M, K in ((4608, 3584), (3584, 3584), (4096, 4096), (1024, 4096), (6144, 4096), (8192, 8192)):
         assert not any(prefers_matrix_cores(r, M, K) for r in range(1, 9)), (M, K)
-    assert [r for r in range(1, 9) if prefers_matrix_cores(r, 3584, 18944)] == [4, 5, 6, 7, 8]
-    assert [r for r in range(1, 9) if prefers_matrix_cores(r, 12288, 4096)] == [6, 7, 8]
-    assert [r for r in range(1, 9) if prefers_matrix_cores(r, 4096, 12288)] == [8]
-    assert not prefers_matrix_cores(8, 3584 + 4, 18944)          # the kernel needs whole blocks of 16 row groups
+    want = {(3584, 18944): [4, 5, 6, 7, 8], (14336, 4096): [4, 5, 6, 7, 8], (18944, 3584): [6, 7, 8],
+            (12288, 4096): [6, 7, 8], (11008, 4096): [6, 7, 8], (4096, 14336): [6, 7, 8],
+            (4096, 12288): [8], (4096, 11008): [8]}
+    for (M, K), rows in want.items():
+        assert [r for r in range(1, 9) if prefers_matrix_cores(r, M, K)] == rows, (M, K)
 
 
 def test_binding_checks_the_member_struct_against_the_library():
