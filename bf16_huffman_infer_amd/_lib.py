@@ -51,6 +51,8 @@ _SIGNATURES = {
     "bhi_silu_mul": (_i32, [_vp, _vp, _vp, _i64, _vp]),
     "bhi_gemm_bf16_huffman": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp, _i64, _vp]),
     "bhi_gemm_bf16_ans": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp, _i64, _vp]),
+    "bhi_gemm_bf16_huffman_grouped": (_i32, [ctypes.POINTER(GemvMember), _i32, _vp, _i32, _i32, _i32, _vp]),
+    "bhi_gemm_bf16_ans_grouped": (_i32, [ctypes.POINTER(GemvMember), _i32, _vp, _i32, _i32, _i32, _vp]),
     "bhi_gemm_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "bhi_gemm_bf16_huffman_static": (_i32, [ctypes.POINTER(GemvMember), _vp, _i32, _i32, _i32, _vp]),
     "bhi_gemm_static_workspace_bytes": (_i64, []),

@@ -161,10 +161,16 @@ extern "C" int bhi_gemv_bf16_ans_grouped_x(const bhi_gemv_member* members, int n
 
 extern "C" int bhi_gemm_bf16_ans(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
                                  void* workspace, int64_t workspace_bytes, void* stream) {
-    if (!weight) return bhi_fail(BHI_EINVAL, "null pointer");
-    if (int rc = launch_mma<AnsCodec>(*weight, X, split_k, Ks, batch, workspace, workspace_bytes, 0, true,
+    if (int rc = launch_mma<AnsCodec>(weight, 1, X, split_k, Ks, batch, workspace, workspace_bytes, 0, true,
                                       (hipStream_t)stream)) return rc;
     return bhi_launch_status("gemm_bf16_ans");
+}
+
+extern "C" int bhi_gemm_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, const void* X, int split_k,
+                                         int Ks, int batch, void* stream) {
+    if (int rc = launch_mma<AnsCodec>(members, n_members, X, split_k, Ks, batch, nullptr, 0, 0, true,
+                                      (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemm_bf16_ans_grouped");
 }
 
 extern "C" int bhi_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_words,

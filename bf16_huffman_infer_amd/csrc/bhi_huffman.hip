@@ -141,10 +141,16 @@ extern "C" int bhi_gemv_bf16_huffman_grouped_x(const bhi_gemv_member* members, i
 
 extern "C" int bhi_gemm_bf16_huffman(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
                                      void* workspace, int64_t workspace_bytes, void* stream) {
-    if (!weight) return bhi_fail(BHI_EINVAL, "null pointer");
-    if (int rc = launch_mma<HuffCodec>(*weight, X, split_k, Ks, batch, workspace, workspace_bytes,
+    if (int rc = launch_mma<HuffCodec>(weight, 1, X, split_k, Ks, batch, workspace, workspace_bytes,
                                        (int64_t)kTableEntries * 4, false, (hipStream_t)stream)) return rc;
     return bhi_launch_status("gemm_bf16_huffman");
+}
+
+extern "C" int bhi_gemm_bf16_huffman_grouped(const bhi_gemv_member* members, int n_members, const void* X, int split_k,
+                                             int Ks, int batch, void* stream) {
+    if (int rc = launch_mma<HuffCodec>(members, n_members, X, split_k, Ks, batch, nullptr, 0,
+                                       (int64_t)kTableEntries * 4, false, (hipStream_t)stream)) return rc;
+    return bhi_launch_status("gemm_bf16_huffman_grouped");
 }
 
 // The workspace of bhi_gemm_bf16_huffman_static: part of the library's image on every GPU
@@ -186,7 +192,7 @@ extern "C" int bhi_gemm_bf16_huffman_static(const bhi_gemv_member* weight, const
                                     "use bhi_gemm_bf16_huffman with a workspace of bhi_gemm_workspace_bytes(...) bytes");
     void* ws = nullptr;
     if (int rc = static_workspace(&ws)) return rc;
-    if (int rc = launch_mma<HuffCodec>(*weight, X, split_k, Ks, batch, ws, kStaticWorkspaceBytes,
+    if (int rc = launch_mma<HuffCodec>(weight, 1, X, split_k, Ks, batch, ws, kStaticWorkspaceBytes,
                                        (int64_t)kTableEntries * 4, false, (hipStream_t)stream)) return rc;
     return bhi_launch_status("gemm_bf16_huffman_static");
 }

@@ -99,11 +99,20 @@ struct MmaArgs {
     const uint32_t* table;
     const uint8_t* header;
     const uint16_t* bias;
+    const uint16_t* residual;
     Shape s;
     int batch;
     int slices;              // K slices (blocks per row block); divides split_k * nc
     float* partial;          // [slices][batch][M] when slices > 1
     uint32_t* counters;      // one per row block, zero between launches
+};
+
+// Up to four weights that multiply the same X in one grid (the gate and up projections of a
+// decoder layer): member i owns the blocks from first[i] on.  Only a group of one is cut
+// along K.
+struct MmaGroup {
+    MmaArgs m[kMaxMembers];
+    int first[kMaxMembers];
 };
 
 // Workspace layout: the arrival counters first, at a fixed place for every shape (a launch
@@ -116,7 +125,7 @@ __host__ __device__ inline long long mma_partial_floats(int M, int batch, int sl
 
 template <class Codec, int Q, int NW>
 __global__ __launch_bounds__(NW * kLanes, mma_resident_blocks(Q, NW) * NW / 4)     // wavefronts per SIMD that the blocks of a compute unit add up to
-void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
+void mma_kernel(const uint16_t* __restrict__ X, int first1, int first2, int first3, const MmaGroup grp) {
     constexpr int S = kMmaSeg;
     constexpr int kWindow = S * Q * kLanes;                   // 16-byte units of one X window
     constexpr int kThreads = NW * kLanes;
@@ -127,10 +136,19 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
     __shared__ uint4 xbuf[2][kWindow];
     __shared__ uint32_t is_last;
 
+    // first1..3: first block of members 1..3 (INT_MAX when absent); leading scalar arguments
+    // are in registers when the wavefront starts, so the member is known without a fetch
+    static_assert(kMaxMembers == 4, "one leading argument per member after the first");
+    int member = 0;
+    if ((int)blockIdx.x >= first1) member = 1;
+    if ((int)blockIdx.x >= first2) member = 2;
+    if ((int)blockIdx.x >= first3) member = 3;
+    const MmaArgs& a = grp.m[member];
+    const int block = (int)blockIdx.x - grp.first[member];
     const Shape s = a.s;
     const int lane = threadIdx.x & (kLanes - 1);
     const int wave = (int)uniform(threadIdx.x / kLanes);
-    const int rb = (int)blockIdx.x / a.slices, ks = (int)blockIdx.x % a.slices;
+    const int rb = block / a.slices, ks = block % a.slices;
     // a block past the last row group (M / 4 need not be a multiple of NW) repeats that group
     // without storing anything: its wavefronts still load their share of X and meet the barriers
     const int G = s.M / kGroupRows;
@@ -250,7 +268,8 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
                 if (batch < B) {
 #pragma unroll
                     for (int i = 0; i < kGroupRows; ++i)
-                        a.Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(pol.acc[q][i], a.bias, kGroupRows * g + i);
+                        a.Y[(size_t)batch * s.M + kGroupRows * g + i] = finish_output(pol.acc[q][i], a.bias, kGroupRows * g + i,
+                                                                                      a.residual ? a.residual + (size_t)batch * s.M : nullptr);
                 }
             }
         }
@@ -298,7 +317,7 @@ void mma_kernel(const uint16_t* __restrict__ X, const MmaArgs a) {
         float v = 0.f;
         for (int k = 0; k < a.slices; ++k)
             v += __hip_atomic_load(a.partial + ((size_t)k * B + batch) * s.M + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        a.Y[(size_t)batch * s.M + row] = finish_output(v, a.bias, row);
+        a.Y[(size_t)batch * s.M + row] = finish_output(v, a.bias, row, a.residual ? a.residual + (size_t)batch * s.M : nullptr);
     }
     if (threadIdx.x == 0) __hip_atomic_store(a.counters + rb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -371,57 +390,83 @@ static inline int64_t mma_workspace_bytes(const bhi::Shape& s, int batch) {
 }
 
 template <class Codec, int Q, int NW>
-static inline void launch_mma_qn(const bhi::MmaArgs& a, const uint16_t* x, hipStream_t stream) {
+static inline void launch_mma_qn(bhi::MmaGroup& grp, int n, const uint16_t* x, hipStream_t stream) {
     using namespace bhi;
-    const int G = a.s.M / kGroupRows;
-    const dim3 grid((unsigned)((G + NW - 1) / NW * a.slices)), block(NW * kLanes);
-    hipLaunchKernelGGL((mma_kernel<Codec, Q, NW>), grid, block, 0, stream, x, a);
+    long long blocks = 0;
+    for (int i = 0; i < kMaxMembers; ++i) {
+        grp.first[i] = i < n ? (int)blocks : 0x7FFFFFFF;
+        if (i < n) blocks += (long long)((grp.m[i].s.M / kGroupRows + NW - 1) / NW) * grp.m[i].slices;
+    }
+    const dim3 grid((unsigned)blocks), block(NW * kLanes);
+    hipLaunchKernelGGL((mma_kernel<Codec, Q, NW>), grid, block, 0, stream, x, grp.first[1], grp.first[2], grp.first[3], grp);
 }
 
 template <class Codec, int Q>
-static inline void launch_mma_q(const bhi::MmaArgs& a, int nw, const uint16_t* x, hipStream_t stream) {
+static inline void launch_mma_q(bhi::MmaGroup& grp, int n, int nw, const uint16_t* x, hipStream_t stream) {
     using namespace bhi;
     if constexpr (Q <= kMmaSmallUpToQ) {
-        if (nw == kMmaWavesSmall) return launch_mma_qn<Codec, Q, kMmaWavesSmall>(a, x, stream);
+        if (nw == kMmaWavesSmall) return launch_mma_qn<Codec, Q, kMmaWavesSmall>(grp, n, x, stream);
     }
-    if (nw == kMmaWavesMid) return launch_mma_qn<Codec, Q, kMmaWavesMid>(a, x, stream);
-    launch_mma_qn<Codec, Q, kMmaWavesLarge>(a, x, stream);
+    if (nw == kMmaWavesMid) return launch_mma_qn<Codec, Q, kMmaWavesMid>(grp, n, x, stream);
+    launch_mma_qn<Codec, Q, kMmaWavesLarge>(grp, n, x, stream);
+}
+
+// The plan of a group is the plan of one weight with all the members' rows.
+static inline bhi::Shape mma_group_shape(const bhi::Shape& first, long long rows) {
+    bhi::Shape s = first;
+    s.M = (int)rows;
+    return s;
 }
 
 template <class Codec>
-static inline int launch_mma(const bhi_gemv_member& m, const void* X, int split_k, int Ks, int batch,
+static inline int launch_mma(const bhi_gemv_member* members, int n_members, const void* X, int split_k, int Ks, int batch,
                              void* workspace, int64_t workspace_bytes, int64_t table_bytes_expected, bool header_is_table,
                              hipStream_t stream) {
     using namespace bhi;
-    if (!X || !m.A_rem || !m.A_exp || !m.Y || !m.offsets || !m.table || (!header_is_table && !m.header))
-        return bhi_fail(BHI_EINVAL, "null pointer");
+    if (!members || !X) return bhi_fail(BHI_EINVAL, "null pointer");
+    if (n_members < 1 || n_members > kMaxMembers) return bhi_fail(BHI_EINVAL, "a group has 1 to 4 members");
     if (batch < 1 || batch > kMmaMaxBatch) return bhi_fail(BHI_EBATCH, "the fused matrix product takes 1 to 32 rows of X");
-    if (table_bytes_expected > 0 && m.table_bytes != table_bytes_expected)
-        return bhi_fail(BHI_ELAYOUT, "decode table has the wrong size");
-    Shape s;
-    if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &s)) return rc;
+    MmaGroup grp = {};
+    long long rows = 0;
+    for (int i = 0; i < n_members; ++i) {
+        const bhi_gemv_member& m = members[i];
+        if (!m.A_rem || !m.A_exp || !m.Y || !m.offsets || !m.table || (!header_is_table && !m.header))
+            return bhi_fail(BHI_EINVAL, "null pointer in a group member");
+        if (table_bytes_expected > 0 && m.table_bytes != table_bytes_expected)
+            return bhi_fail(BHI_ELAYOUT, "decode table has the wrong size");
+        MmaArgs& a = grp.m[i];
+        if (int rc = check_shape(split_k, m.M, Ks, m.exp_words, &a.s)) return rc;
+        a.rem = (const uint8_t*)m.A_rem; a.exp = (const uint32_t*)m.A_exp; a.Y = (uint16_t*)m.Y;
+        a.offsets = (const uint32_t*)m.offsets; a.table = (const uint32_t*)m.table;
+        a.header = (const uint8_t*)(header_is_table ? m.table : m.header); a.bias = (const uint16_t*)m.bias;
+        a.residual = (const uint16_t*)m.residual;
+        a.batch = batch; a.slices = 1;
+        a.counters = nullptr; a.partial = nullptr;
+        rows += m.M;
+    }
+    if (rows > 0x7FFFFFFFll) return bhi_fail(BHI_EINVAL, "group too large for one launch");
     const int Q = (batch + 3) / 4;
-    const MmaPlan plan = mma_plan(s, Q);
-    const int slices = plan.slices;
-    const int64_t need = mma_workspace_bytes(s, batch);
-    if (slices > 1 && (!workspace || workspace_bytes < need)) return bhi_fail(BHI_EINVAL, "workspace too small: see bhi_gemm_workspace_bytes");
-    MmaArgs a;
-    a.rem = (const uint8_t*)m.A_rem; a.exp = (const uint32_t*)m.A_exp; a.Y = (uint16_t*)m.Y;
-    a.offsets = (const uint32_t*)m.offsets; a.table = (const uint32_t*)m.table;
-    a.header = (const uint8_t*)(header_is_table ? m.table : m.header); a.bias = (const uint16_t*)m.bias;
-    a.s = s; a.batch = batch; a.slices = slices;
-    a.counters = (uint32_t*)workspace;
-    a.partial = (float*)((char*)workspace + kMmaCounterBytes);
+    const Shape whole = mma_group_shape(grp.m[0].s, rows);
+    const MmaPlan plan = mma_plan(whole, Q);
+    if (plan.slices > 1) {
+        if (n_members > 1)
+            return bhi_fail(BHI_EINVAL, "a group this small would be cut along K: launch its members one by one");
+        const int64_t need = mma_workspace_bytes(whole, batch);
+        if (!workspace || workspace_bytes < need) return bhi_fail(BHI_EINVAL, "workspace too small: see bhi_gemm_workspace_bytes");
+        grp.m[0].slices = plan.slices;
+        grp.m[0].counters = (uint32_t*)workspace;
+        grp.m[0].partial = (float*)((char*)workspace + kMmaCounterBytes);
+    }
     const uint16_t* x = (const uint16_t*)X;
     switch (Q) {
-        case 1: launch_mma_q<Codec, 1>(a, plan.nw, x, stream); break;
-        case 2: launch_mma_q<Codec, 2>(a, plan.nw, x, stream); break;
-        case 3: launch_mma_q<Codec, 3>(a, plan.nw, x, stream); break;
-        case 4: launch_mma_q<Codec, 4>(a, plan.nw, x, stream); break;
-        case 5: launch_mma_q<Codec, 5>(a, plan.nw, x, stream); break;
-        case 6: launch_mma_q<Codec, 6>(a, plan.nw, x, stream); break;
-        case 7: launch_mma_q<Codec, 7>(a, plan.nw, x, stream); break;
-        default: launch_mma_q<Codec, 8>(a, plan.nw, x, stream); break;
+        case 1: launch_mma_q<Codec, 1>(grp, n_members, plan.nw, x, stream); break;
+        case 2: launch_mma_q<Codec, 2>(grp, n_members, plan.nw, x, stream); break;
+        case 3: launch_mma_q<Codec, 3>(grp, n_members, plan.nw, x, stream); break;
+        case 4: launch_mma_q<Codec, 4>(grp, n_members, plan.nw, x, stream); break;
+        case 5: launch_mma_q<Codec, 5>(grp, n_members, plan.nw, x, stream); break;
+        case 6: launch_mma_q<Codec, 6>(grp, n_members, plan.nw, x, stream); break;
+        case 7: launch_mma_q<Codec, 7>(grp, n_members, plan.nw, x, stream); break;
+        default: launch_mma_q<Codec, 8>(grp, n_members, plan.nw, x, stream); break;
     }
     return 0;
 }

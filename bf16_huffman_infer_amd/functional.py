@@ -20,6 +20,7 @@ from .ans import RANSEncoder
 from .huffman import LUTHuffmanEncoder
 from . import ops as _ops
 from .ops import (GEMM_MAX_ROWS, ans_decode, ans_encode, ans_encode_capacity, encode_capacity, gemm_bf16,
+                  gemm_bf16_grouped,
                   gemv_bf16_ans, gemv_bf16_grouped, gemv_bf16_huffman, gemv_bf16_nibble, huffman_decode, huffman_encode,
                   nibble_decode, nibble_encode, nibble_encode_capacity)
 from .utils import get_block_size_n, split_bf16
@@ -453,13 +454,12 @@ def linear_grouped(input: Tensor, weights, biases=None, *, residuals=None, input
         biases = [None if b is None else b.detach().contiguous() for b in biases]
     if residuals is not None:
         residuals = [None if r is None else r.detach().reshape(x.size(0), -1).contiguous() for r in residuals]
-    if (mode == _ops.X_PLAIN and (residuals is None or all(r is None for r in residuals))
-            and not isinstance(first, NibbleWeight)
-            and all(prefers_matrix_cores(x.size(0), w.rem.shape[1], split_k * N) for w in weights)):
-        # layers this large are faster through the matrix-core kernel, one launch per member
-        x = x.contiguous()
-        for i, (w, y) in enumerate(zip(weights, ys)):
-            gemm_bf16(w, x, y, None if biases is None else biases[i])
+    total = sum(w.rem.shape[1] for w in weights)
+    if (mode == _ops.X_PLAIN and not isinstance(first, NibbleWeight)
+            and (all(prefers_matrix_cores(x.size(0), w.rem.shape[1], split_k * N) for w in weights)
+                 or prefers_matrix_cores(x.size(0), total, split_k * N))):
+        # layers this large -- or this large together -- are faster through the matrix-core kernel
+        gemm_bf16_grouped(weights, x.contiguous(), ys, biases, residuals)
     else:
         gemv_bf16_grouped(weights, x.contiguous(), ys, biases, residuals, mode, aux, float(eps))
     return [y.unflatten(0, shape[:-1]) for y in ys]

@@ -426,13 +426,14 @@ def _gemm_workspace(device: torch.device, stream: int, nbytes: int, allocate=Non
     return held[-1]
 
 
-def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None, static_workspace: bool = False) -> None:
+def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None, static_workspace: bool = False, residual=None) -> None:
     """``Y = X @ W.T (+ bias)`` for up to 32 rows of ``X`` with ``W`` held compressed
     (:class:`HuffmanWeight` or :class:`ANSWeight`), decoded inside the matrix-core kernel.
 
     Takes the place of ``get_weight()`` + ``F.linear`` in the reference's path above eight
     rows (``functional.py:405-407, 460-462``).  ``X`` bf16 ``[rows, split_k, Ks]``, ``Y`` bf16
-    ``[rows, M]`` written.  Plain function: only enqueues on the current stream.  Products that
+    ``[rows, M]`` written; ``bias`` (bf16 ``[M]``) and then ``residual`` (bf16 ``[rows, M]``) are added
+    as separate BF16 additions would.  Plain function: only enqueues on the current stream.  Products that
     are cut along K keep their partial sums in a workspace that belongs to the (device, stream)
     pair of the call and is allocated (and zeroed by a fill kernel) at the first such call on
     that stream -- also under stream capture, where the allocation comes from the graph's own
@@ -449,6 +450,10 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None, static_workspace: bool = 
     member = (_lib.GemvMember * 1)()
     x_ptr = _req(X, torch.bfloat16, "X", weight.rem)
     huffman = _fill_member(member[0], weight, Y, bias, weight.rem)
+    if residual is not None:
+        if tuple(residual.shape) != (rows, M):
+            raise RuntimeError(f"residual must be [{rows}, {M}], got {tuple(residual.shape)}")
+        member[0].residual = _req(residual, torch.bfloat16, "residual", weight.rem)
     name = "gemm_bf16_huffman" if huffman else "gemm_bf16_ans"
     device = weight.rem.device
     stream = _stream(weight.rem)
@@ -471,6 +476,49 @@ def gemm_bf16(weight, X: Tensor, Y: Tensor, bias=None, static_workspace: bool = 
         if rc != 0 and ws is not None:
             # the launch did not happen or was cut short: its counters may not be zero any more
             lib.bhi_gemm_workspace_reset(ws.data_ptr(), ws.numel(), stream)
+    _lib.check(rc, name)
+
+
+def gemm_bf16_grouped(weights, X: Tensor, Ys, biases=None, residuals=None) -> None:
+    """:func:`gemm_bf16` for up to four weights of one class (Huffman or rANS) and one ``split_k`` / ``Ks``
+    that multiply the same ``X``: one grid when their rows together are enough for the kernel to
+    run without cutting along K (8192 rows), else one launch per member.  Stands in, like
+    :func:`gemv_bf16_grouped`, for the reference's parallel streams (``cudastream_utils.py:8-47``)."""
+    n = len(weights)
+    if not 1 <= n <= 4 or n != len(Ys):
+        raise RuntimeError("a group has 1 to 4 weights and one output per weight")
+    biases = [None] * n if biases is None else list(biases)
+    residuals = [None] * n if residuals is None else list(residuals)
+    first = weights[0]
+    split_k, _, Ks = _weight_dims(first.rem, first.offsets)
+    if X.dim() != 3 or X.shape[1] != split_k or X.shape[2] != Ks:
+        raise RuntimeError(f"X must be [rows, {split_k}, {Ks}], got {tuple(X.shape)}")
+    rows = X.shape[0]
+    dims = [_weight_dims(w.rem, w.offsets) for w in weights]
+    if any(type(w) is not type(first) for w in weights):
+        raise RuntimeError("the weights of a group must use one codec")
+    if any((sk, ks) != (split_k, Ks) for sk, _, ks in dims):
+        raise RuntimeError("the weights of a group must share split_k and Ks")
+    lib = _lib.load()
+    total = sum(M for _, M, _ in dims)
+    if n == 1 or int(lib.bhi_gemm_workspace_bytes(split_k, total, Ks, rows)) != 0:
+        for w, Y, b, r in zip(weights, Ys, biases, residuals):
+            gemm_bf16(w, X, Y, b, residual=r)
+        return
+    members = (_lib.GemvMember * n)()
+    x_ptr = _req(X, torch.bfloat16, "X", first.rem)
+    huffman = True
+    for m, w, (_, M, _), Y, b, r in zip(members, weights, dims, Ys, biases, residuals):
+        if tuple(Y.shape) != (rows, M):
+            raise RuntimeError(f"Y must be [{rows}, {M}], got {tuple(Y.shape)}")
+        huffman = _fill_member(m, w, Y, b, first.rem)
+        if r is not None:
+            if tuple(r.shape) != (rows, M):
+                raise RuntimeError(f"residual must be [{rows}, {M}], got {tuple(r.shape)}")
+            m.residual = _req(r, torch.bfloat16, "residual", first.rem)
+    name = "gemm_bf16_huffman_grouped" if huffman else "gemm_bf16_ans_grouped"
+    with torch.cuda.device(first.rem.device):
+        rc = getattr(lib, "bhi_" + name)(members, n, x_ptr, split_k, Ks, rows, _stream(first.rem))
     _lib.check(rc, name)
 
 

@@ -187,7 +187,7 @@ int bhi_silu_mul(const void* gate, const void* up, void* out, int64_t n, void* s
  * eight rows, huffman_decode / ans_decode to a BF16 matrix followed by a dense GEMM
  * (functional.py:405-407, 460-462; kernel.cu:510-587, 851-919), which writes and re-reads
  * 2*M*K bytes per call.  `weight` is one member as the grouped GEMV takes it (Y bf16
- * [batch, M]; M a multiple of 64).  Weights with fewer than 2048 row groups are cut along K
+ * [batch, M]; bias and residual as there).  Weights with fewer than 2048 row groups are cut along K
  * over several blocks whose partial sums meet in `workspace`: device memory of at least
  * bhi_gemm_workspace_bytes(...) bytes that was ZERO when first handed to the library and is
  * otherwise only touched by these entry points (every launch leaves its counters at zero);
@@ -197,6 +197,16 @@ int bhi_gemm_bf16_huffman(const bhi_gemv_member* weight, const void* X, int spli
                           void* workspace, int64_t workspace_bytes, void* stream);
 int bhi_gemm_bf16_ans(const bhi_gemv_member* weight, const void* X, int split_k, int Ks, int batch,
                       void* workspace, int64_t workspace_bytes, void* stream);
+/* The same product for up to four weights that multiply one X (members as in the grouped GEMV:
+ * same codec, split_k and Ks; bias and residual per member), one grid -- what the reference
+ * spreads over parallel streams for the sibling projections of a decoder layer
+ * (cudastream_utils.py:8-47).  Takes no workspace: a group whose rows together number fewer
+ * than 8192 (bhi_gemm_workspace_bytes of the summed M is not 0) is rejected with BHI_EINVAL and
+ * its members go through the calls above one by one. */
+int bhi_gemm_bf16_huffman_grouped(const bhi_gemv_member* members, int n_members, const void* X, int split_k,
+                                  int Ks, int batch, void* stream);
+int bhi_gemm_bf16_ans_grouped(const bhi_gemv_member* members, int n_members, const void* X, int split_k,
+                              int Ks, int batch, void* stream);
 /* Workspace bytes a call with these dimensions needs (0: none); negative on a rejected shape. */
 int64_t bhi_gemm_workspace_bytes(int split_k, int M, int Ks, int batch);
 

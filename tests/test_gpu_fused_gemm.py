@@ -81,6 +81,57 @@ def test_row_counts_that_fill_no_whole_block(cuda, algo, rows, M, K):
     assert bool((guard == 7.0).all())
 
 
+@pytest.mark.parametrize("algo", ["huffman", "ans"])
+@pytest.mark.parametrize("rows", [3, 16, 32])
+@pytest.mark.parametrize("Ms", [(2048, 4096, 2560), (1024, 1024, 1024), (8192, 8320)])
+def test_grouped_product(cuda, algo, rows, Ms):
+    """Up to four weights in one grid (8704 and 16512 rows: the grouped entry point; 3072 rows: too few,
+    one launch per member), with a bias on one member and a residual on another: against fp32, and bit
+    for bit against the members' own launches where those are not cut along K either."""
+    from bf16_huffman_infer_amd import _lib, ops
+    K = 1024
+    ws = [gaussian_weight(M, K, seed=60 + i) for i, M in enumerate(Ms)]
+    mods = [_cls(algo).compress(w).cuda() for w in ws]
+    x = torch.randn(rows, K, generator=torch.Generator().manual_seed(rows)).bfloat16().cuda()
+    x3 = x.view(rows, *mods[0].rem.shape[::2])
+    biases = [None] * len(Ms)
+    biases[0] = (torch.randn(Ms[0], generator=torch.Generator().manual_seed(1)) * 0.1).bfloat16().cuda()
+    residuals = [None] * len(Ms)
+    residuals[-1] = torch.randn(rows, Ms[-1], generator=torch.Generator().manual_seed(2)).bfloat16().cuda()
+    ys = [torch.full((rows, M), float("nan"), dtype=torch.bfloat16, device="cuda") for M in Ms]
+    ops.gemm_bf16_grouped(mods, x3, ys, biases, residuals)
+    for w, mod, b, r, y in zip(ws, mods, biases, residuals, ys):
+        want = (x.float() @ w.cuda().float().T).bfloat16()
+        if b is not None:
+            want = want + b
+        if r is not None:
+            want = want + r
+        torch.testing.assert_close(y.float(), want.float(), rtol=RTOL, atol=ATOL + 2.0 ** -7 * want.float().abs().max().item())
+        sk, M, Ks = mod.rem.shape
+        if _lib.load().bhi_gemm_workspace_bytes(sk, M, Ks, rows) == 0:
+            single = torch.empty_like(y)
+            ops.gemm_bf16(mod, x3, single, b, residual=r)
+            assert torch.equal(single.view(torch.int16), y.view(torch.int16))
+
+
+def test_grouped_product_rejections(cuda):
+    from bf16_huffman_infer_amd import _lib, ops
+    w = gaussian_weight(1024, 1024, seed=3)
+    a, b = _cls("huffman").compress(w).cuda(), _cls("ans").compress(w).cuda()
+    x = torch.randn(16, 1, 1024).bfloat16().cuda()
+    ys = [torch.empty(16, 1024, dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+    with pytest.raises(RuntimeError, match="one codec"):
+        ops.gemm_bf16_grouped([a, b], x, ys)
+    with pytest.raises(RuntimeError, match="1 to 4"):
+        ops.gemm_bf16_grouped([a] * 5, x, ys * 3)
+    # the C entry point refuses a group it would have to cut along K
+    members = (_lib.GemvMember * 2)()
+    for m, y in zip(members, ys):
+        ops._fill_member(m, a, y, None, a.rem)
+    rc = _lib.load().bhi_gemm_bf16_huffman_grouped(members, 2, x.data_ptr(), 1, 1024, 16, None)
+    assert rc != 0 and b"one by one" in _lib.load().bhi_last_error_string()
+
+
 def test_more_than_32_rows_still_decode_then_gemm(cuda):
     w = gaussian_weight(256, 512, seed=7)
     mod = _cls("huffman").compress(w).cuda()
