@@ -472,8 +472,10 @@ class LinearGroup:
     The call of the first member computes every member's output in one grouped launch
     and keeps the others until their own call collects them.  Whatever does not fit that
     pattern -- more than 8 rows, a member called alone or on another tensor, weights of
-    different codecs or splits -- runs each member's ordinary path, so grouping never
-    changes results, only the number of launches.
+    different codecs or splits -- runs each member's ordinary path.  Grouping changes the
+    number of launches and, where members that are large only together move to the matrix-core
+    kernel (:func:`prefers_matrix_cores`), the order of the fp32 sums: a last bit of BF16 here
+    and there, nothing else.
     """
 
     def __init__(self, members):
@@ -682,13 +684,18 @@ def prefers_matrix_cores(rows: int, M: int, K: int) -> bool:
     ===========  ===========  ===========  ===========  ===========
 
     and the layers of 6144x4096 and below are 0.4-4 us faster on the GEMV at every row count; output
-    layers the size of a vocabulary are faster on the matrix cores from 4 rows (152064x3584:
-    180 / 148, 202 / 184, 225 / 185 us at 4, 6, 8 rows; 37888x3584: 44.4 / 39.8, 52.2 / 48.7, 58.7 / 48.9)."""
+    layers the size of a vocabulary -- or a group of layers that large together -- are faster on the
+    matrix cores from 3 rows (152064x3584: 138 / 147, 157 / 148, 180 / 148, 225 / 185 us at 2, 3, 4, 8
+    rows; 37888x3584: 39.1 / 39.6, 41.9 / 39.7, 44.4 / 39.8, 58.7 / 48.9).  The rANS kernels cross over
+    at the same places (18944x3584 at 6 rows 37.7 / 36.0, 3584x18944 at 4 rows 34.7 / 33.9,
+    37888x3584 at 3 rows 53.6 / 51.2)."""
     if rows >= 8 and K >= 11008:
         return True
     if rows >= 6 and ((M >= 10240 and K >= 3584) or K >= 14336):
         return True
-    return rows >= 4 and (K >= 16384 or (M >= 14336 and K >= 4096) or (M >= 32768 and K >= 3584))
+    if rows >= 4 and (K >= 16384 or (M >= 14336 and K >= 4096)):
+        return True
+    return rows >= 3 and M >= 32768 and K >= 3584
 
 
 def _linear_compressed(input: Tensor, weight: HuffmanWeight, bias: Optional[Tensor], fused) -> Tensor:

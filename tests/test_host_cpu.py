@@ -106,7 +106,7 @@ def test_dispatch_rule_between_gemv_and_matrix_cores():
         assert not any(prefers_matrix_cores(r, M, K) for r in range(1, 9)), (M, K)
     want = {(3584, 18944): [4, 5, 6, 7, 8], (14336, 4096): [4, 5, 6, 7, 8], (18944, 3584): [6, 7, 8],
             (12288, 4096): [6, 7, 8], (11008, 4096): [6, 7, 8], (4096, 14336): [6, 7, 8],
-            (4096, 12288): [8], (4096, 11008): [8]}
+            (4096, 12288): [8], (4096, 11008): [8], (37888, 3584): [3, 4, 5, 6, 7, 8], (152064, 3584): [3, 4, 5, 6, 7, 8]}
     for (M, K), rows in want.items():
         assert [r for r in range(1, 9) if prefers_matrix_cores(r, M, K)] == rows, (M, K)
 
