@@ -47,19 +47,20 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 #define BHI_MMA_LAST_ACQUIRES 1
 #endif
 constexpr int kMmaSeg = 4;                   // steps per window
-// Wavefronts (row groups) per block.  LDS holds two windows of X (8 KB per batch quad) beside
-// the table and the rings: up to 16 rows two 8-wavefront blocks fit a compute unit, and one
-// block of 12 or of 16 at any batch.  Which one a launch takes is a matter of how evenly its
-// blocks cover the 256 compute units (mma_plan below).
+constexpr int kMmaSegShort = 2;              // at 5..8 rows also built with short windows: 8 KB less LDS, a third block per unit
+// Wavefronts (row groups) per block.  LDS holds two windows of X (8 KB per batch quad, half of
+// that with short windows) beside the table and the rings: up to 16 rows two 8-wavefront blocks
+// fit a compute unit, and one block of 12 or of 16 at any batch.  Which one a launch takes is
+// a matter of how evenly its blocks cover the 256 compute units (mma_plan below).
 constexpr int kMmaWavesSmall = 8, kMmaWavesMid = 12, kMmaWavesLarge = 16;
 constexpr int kMmaSmallUpToQ = 4;            // 8-wavefront blocks: batch quads 1..4
-// Blocks of NW wavefronts that a compute unit holds at Q batch quads: by LDS (rings 4.5 KB per
-// wavefront, table up to 8 KB, X windows 8 KB per quad, 160 KB per unit) and by registers
-// (65-73 up to two quads: six wavefronts per SIMD; 84-102 up to four quads: four; above: three
-// or four)
-constexpr int mma_resident_blocks(int Q, int NW) {
+// Blocks of NW wavefronts that a compute unit holds at Q batch quads and windows of S steps:
+// by LDS (rings 4.5 KB per wavefront, table up to 8 KB, X windows 2 KB per quad and step,
+// 160 KB per unit) and by registers (65-73 up to two quads: six wavefronts per SIMD; 84-102 up
+// to four quads: four; above: three or four)
+constexpr int mma_resident_blocks(int Q, int NW, int S = kMmaSeg) {
     return Q == 1 ? (NW == kMmaWavesSmall ? 3 : (NW == kMmaWavesMid ? 2 : 1))
-         : Q == 2 ? (NW == kMmaWavesLarge ? 1 : 2)
+         : Q == 2 ? (NW == kMmaWavesLarge ? 1 : (NW == kMmaWavesSmall && S == kMmaSegShort ? 3 : 2))
          : Q <= 4 ? (NW == kMmaWavesSmall ? 2 : 1) : 1;
 }
 constexpr int kMmaMaxBatch = 32;
@@ -123,10 +124,9 @@ __host__ __device__ inline long long mma_partial_floats(int M, int batch, int sl
     return slices > 1 ? (long long)slices * batch * M : 0;
 }
 
-template <class Codec, int Q, int NW>
-__global__ __launch_bounds__(NW * kLanes, mma_resident_blocks(Q, NW) * NW / 4)     // wavefronts per SIMD that the blocks of a compute unit add up to
+template <class Codec, int Q, int NW, int S = kMmaSeg>
+__global__ __launch_bounds__(NW * kLanes, mma_resident_blocks(Q, NW, S) * NW / 4)     // wavefronts per SIMD that the blocks of a compute unit add up to
 void mma_kernel(const uint16_t* __restrict__ X, int first1, int first2, int first3, const MmaGroup grp) {
-    constexpr int S = kMmaSeg;
     constexpr int kWindow = S * Q * kLanes;                   // 16-byte units of one X window
     constexpr int kThreads = NW * kLanes;
     constexpr int kPieces = S * Q * 4 * 16;                   // 16-byte pieces of a window: (step, batch row, 8 columns)
@@ -340,13 +340,16 @@ void mma_kernel(const uint16_t* __restrict__ X, int first1, int first2, int firs
 // blocks of 12).  Blocks beyond what is resident at once wait for a round; the last round runs
 // at the pace of the wavefronts it puts on a unit (18944x3584 at 16 rows, 592 blocks of 8:
 // 38.1 us, 395 blocks of 12: 39.5 us; at 8 rows, where two blocks of 12 fit a unit: 31.0 and
-// 26.3 us).  The 8-wavefront block (16 above 16 rows) stays unless another shape is at least
+// 26.3 us).  At 5..8 rows the 8-wavefront block also comes with windows of two steps: a third
+// block fits the unit and every step costs about 3 % more (37888x3584: 49.0 -> 45.1 us;
+// 3584x18944, whose 448 blocks have room anyway: 28.8 -> 30.9 us).
+// The 8-wavefront block (16 above 16 rows) stays unless another shape is at least
 // 4 % cheaper, and so does a smaller number of slices: the model is no more exact than that.
 // It reproduces the order measured at 16 / 32 rows for the slices as well: 4096x12288
 // (6 tasks of 16 steps) 2 slices 32 us, 3 slices 33 us, 6 slices 41 us, none 50 us / 3 slices
 // 44 us, 2 slices 55 us, 6 slices 59 us; 3584x18944 (4 tasks of 37 steps) 4 slices 36 us,
 // 2 slices 42 us; 4096x4096 (4 tasks of 8 steps) 2 slices 17 us, 4 slices 20 us.
-struct MmaPlan { int nw, slices; };
+struct MmaPlan { int nw, slices, seg; };
 
 // time of a row group on a unit that holds `waves` wavefronts, relative to a lone block of 8
 static inline double mma_pace(int waves) {
@@ -359,15 +362,19 @@ static inline MmaPlan mma_plan(const bhi::Shape& s, int Q) {
     const int G = s.M / kGroupRows, per_group = s.split_k * s.nc;
     const double task_steps = (double)s.steps / s.nc;
     const int max_slices = G >= kMmaSliceBelowGroups ? 1 : kMmaMaxSlices;
-    MmaPlan best = {0, 1};
+    MmaPlan best = {0, 1, kMmaSeg};
     double best_cost = 0;
     const bool small = Q <= kMmaSmallUpToQ;
-    const int candidates[3] = {small ? kMmaWavesSmall : kMmaWavesLarge, kMmaWavesMid, small ? kMmaWavesLarge : 0};
-    for (int nw : candidates) {
+    struct Candidate { int nw, seg; };
+    const Candidate candidates[4] = {{small ? kMmaWavesSmall : kMmaWavesLarge, kMmaSeg}, {kMmaWavesMid, kMmaSeg},
+                                     {small ? kMmaWavesLarge : 0, kMmaSeg}, {Q == 2 ? kMmaWavesSmall : 0, kMmaSegShort}};
+    for (const Candidate& c : candidates) {
+        const int nw = c.nw;
         if (nw == 0) continue;
         const long long row_blocks = (G + nw - 1) / nw;
-        const int resident = mma_resident_blocks(Q, nw);
-        MmaPlan here = {nw, 1};
+        const int resident = mma_resident_blocks(Q, nw, c.seg);
+        const double step_cost = c.seg == kMmaSeg ? 1.0 : 1.03;
+        MmaPlan here = {nw, 1, c.seg};
         double here_cost = 0;
         for (int d = 1; d <= max_slices && d <= per_group; ++d) {
             if (per_group % d != 0) continue;
@@ -375,8 +382,8 @@ static inline MmaPlan mma_plan(const bhi::Shape& s, int Q) {
             const long long rest = blocks % (256 * resident);
             double pace = mma_pace(nw * resident) * (double)(blocks / (256 * resident));
             if (rest > 0) pace += mma_pace(nw * (int)((rest + 255) / 256));
-            const double cost = pace * (per_group / d * task_steps + 6.0) + 2.0 * d;
-            if (d == 1 || cost < 0.96 * here_cost) { here = MmaPlan{nw, d}; here_cost = cost; }
+            const double cost = step_cost * pace * (per_group / d * task_steps + 6.0) + 2.0 * d;
+            if (d == 1 || cost < 0.96 * here_cost) { here = MmaPlan{nw, d, c.seg}; here_cost = cost; }
         }
         if (best.nw == 0 || here_cost < 0.96 * best_cost) { best = here; best_cost = here_cost; }
     }
@@ -389,7 +396,7 @@ static inline int64_t mma_workspace_bytes(const bhi::Shape& s, int batch) {
     return slices > 1 ? kMmaCounterBytes + mma_partial_floats(s.M, batch, slices) * 4 : 0;
 }
 
-template <class Codec, int Q, int NW>
+template <class Codec, int Q, int NW, int S = bhi::kMmaSeg>
 static inline void launch_mma_qn(bhi::MmaGroup& grp, int n, const uint16_t* x, hipStream_t stream) {
     using namespace bhi;
     long long blocks = 0;
@@ -398,12 +405,16 @@ static inline void launch_mma_qn(bhi::MmaGroup& grp, int n, const uint16_t* x, h
         if (i < n) blocks += (long long)((grp.m[i].s.M / kGroupRows + NW - 1) / NW) * grp.m[i].slices;
     }
     const dim3 grid((unsigned)blocks), block(NW * kLanes);
-    hipLaunchKernelGGL((mma_kernel<Codec, Q, NW>), grid, block, 0, stream, x, grp.first[1], grp.first[2], grp.first[3], grp);
+    hipLaunchKernelGGL((mma_kernel<Codec, Q, NW, S>), grid, block, 0, stream, x, grp.first[1], grp.first[2], grp.first[3], grp);
 }
 
 template <class Codec, int Q>
-static inline void launch_mma_q(bhi::MmaGroup& grp, int n, int nw, const uint16_t* x, hipStream_t stream) {
+static inline void launch_mma_q(bhi::MmaGroup& grp, int n, const MmaPlan& plan, const uint16_t* x, hipStream_t stream) {
     using namespace bhi;
+    const int nw = plan.nw;
+    if constexpr (Q == 2) {
+        if (plan.seg == kMmaSegShort) return launch_mma_qn<Codec, Q, kMmaWavesSmall, kMmaSegShort>(grp, n, x, stream);
+    }
     if constexpr (Q <= kMmaSmallUpToQ) {
         if (nw == kMmaWavesSmall) return launch_mma_qn<Codec, Q, kMmaWavesSmall>(grp, n, x, stream);
     }
@@ -459,14 +470,14 @@ static inline int launch_mma(const bhi_gemv_member* members, int n_members, cons
     }
     const uint16_t* x = (const uint16_t*)X;
     switch (Q) {
-        case 1: launch_mma_q<Codec, 1>(grp, n_members, plan.nw, x, stream); break;
-        case 2: launch_mma_q<Codec, 2>(grp, n_members, plan.nw, x, stream); break;
-        case 3: launch_mma_q<Codec, 3>(grp, n_members, plan.nw, x, stream); break;
-        case 4: launch_mma_q<Codec, 4>(grp, n_members, plan.nw, x, stream); break;
-        case 5: launch_mma_q<Codec, 5>(grp, n_members, plan.nw, x, stream); break;
-        case 6: launch_mma_q<Codec, 6>(grp, n_members, plan.nw, x, stream); break;
-        case 7: launch_mma_q<Codec, 7>(grp, n_members, plan.nw, x, stream); break;
-        default: launch_mma_q<Codec, 8>(grp, n_members, plan.nw, x, stream); break;
+        case 1: launch_mma_q<Codec, 1>(grp, n_members, plan, x, stream); break;
+        case 2: launch_mma_q<Codec, 2>(grp, n_members, plan, x, stream); break;
+        case 3: launch_mma_q<Codec, 3>(grp, n_members, plan, x, stream); break;
+        case 4: launch_mma_q<Codec, 4>(grp, n_members, plan, x, stream); break;
+        case 5: launch_mma_q<Codec, 5>(grp, n_members, plan, x, stream); break;
+        case 6: launch_mma_q<Codec, 6>(grp, n_members, plan, x, stream); break;
+        case 7: launch_mma_q<Codec, 7>(grp, n_members, plan, x, stream); break;
+        default: launch_mma_q<Codec, 8>(grp, n_members, plan, x, stream); break;
     }
     return 0;
 }
