@@ -65,25 +65,48 @@ class Block(nn.Module):
 
     fused = False            # set by fuse_neighbours() once every projection is compressed
 
-    def forward(self, x, pos, cos, sin, visible, k_cache, v_cache):
+    kernel_attention = True  # the library's one-launch attention step; False: the same step in torch operations
+
+    def attend(self, qk, v, pos, rot, k_cache, v_cache):
+        """Per-head RMSNorm and rotary embedding of q and k ([q_heads + kv_heads, head_dim], as
+        projected), cache update at ``pos``, attention of the one query over the visible slots.
+        ``rot = (cos, sin, hidden, cos_table, sin_table)``: this position's cosines and signed
+        sines for every head (the softmax scale already in the q rows) and 0 / -inf over the cache
+        slots, all fp32 and computed once per token, and the tables they were taken from.
+        Scores and softmax in fp32; the four query heads that share a key/value head form one
+        matrix product with it (no expanded copies of the cache)."""
+        c = self.c
+        cos, sin, hidden, cos_table, sin_table = rot
+        if self.kernel_attention and qk.is_cuda and c.head_dim == 128:
+            from bf16_huffman_infer_amd.ops import decode_attention
+            return decode_attention(qk, v.view(c.kv_heads, c.head_dim), self.qk_norm, cos_table, sin_table, pos,
+                                    k_cache, v_cache, eps=c.eps).view(1, c.q_heads * c.head_dim)
+        x = F.rms_norm(qk.float(), (c.head_dim,), None, c.eps) * self.qk_norm
+        turned = x.view(-1, 2, c.head_dim // 2).flip(1).view(-1, c.head_dim)       # (x1, x2) -> (x2, x1)
+        x = torch.addcmul(x * cos, turned, sin).to(qk.dtype)
+        k_cache.index_copy_(1, pos, x[c.q_heads:, None, :])                          # [kv, max_len, d]
+        v_cache.index_copy_(1, pos, v.view(c.kv_heads, 1, c.head_dim))
+        q = x[:c.q_heads].view(c.kv_heads, c.q_heads // c.kv_heads, c.head_dim)
+        if q.is_cuda:
+            scores = torch.bmm(q, k_cache.transpose(1, 2), out_dtype=torch.float32) + hidden
+        else:
+            scores = torch.bmm(q.float(), k_cache.float().transpose(1, 2)) + hidden
+        weights = torch.softmax(scores, -1).to(qk.dtype)
+        return torch.bmm(weights, v_cache).view(1, c.q_heads * c.head_dim)
+
+    def forward(self, x, pos, rot, k_cache, v_cache):
         c = self.c
         if self.fused:
-            return self.forward_fused(x, pos, cos, sin, visible, k_cache, v_cache)
+            return self.forward_fused(x, pos, rot, k_cache, v_cache)
         h = rms_norm(x, self.input_norm, c.eps)
         qk = torch.cat((self.q_proj(h), self.k_proj(h)), -1).view(c.q_heads + c.kv_heads, c.head_dim)
-        v = self.v_proj(h).view(c.kv_heads, 1, c.head_dim)
-        qk = rope(F.rms_norm(qk, (c.head_dim,), None, c.eps) * self.qk_norm, cos, sin)
-        q, k = qk[:c.q_heads], qk[c.q_heads:]
-        k_cache.index_copy_(1, pos, k[:, None, :])                      # [kv, max_len, d]
-        v_cache.index_copy_(1, pos, v)
-        a = F.scaled_dot_product_attention(q[None, :, None, :], k_cache[None], v_cache[None],
-                                           attn_mask=visible, enable_gqa=True)      # [1, q, 1, d]
-        x = x + self.o_proj(a.reshape(1, c.q_heads * c.head_dim))
+        a = self.attend(qk, self.v_proj(h), pos, rot, k_cache, v_cache)
+        x = x + self.o_proj(a)
         h = rms_norm(x, self.post_norm, c.eps)
         return x + self.down_proj(F.silu(self.gate_proj(h)) * self.up_proj(h))
 
 
-def _forward_fused(self, x, pos, cos, sin, visible, k_cache, v_cache):
+def _forward_fused(self, x, pos, rot, k_cache, v_cache):
     """The same layer with the pieces next to a linear inside its launch: the RMSNorm in front of
     q/k/v, silu(gate) * up in front of down_proj, both residual additions behind o_proj and
     down_proj, q and k written side by side (no concatenation).  The RMSNorm in front of gate/up
@@ -96,15 +119,8 @@ def _forward_fused(self, x, pos, cos, sin, visible, k_cache, v_cache):
     v = torch.empty(1, nk, dtype=x.dtype, device=x.device)
     linear_grouped(x, [self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], input_norm=(self.input_norm, c.eps),
                    outs=[qk[:, :nq], qk[:, nq:], v])
-    qk = qk.view(c.q_heads + c.kv_heads, c.head_dim)
-    v = v.view(c.kv_heads, 1, c.head_dim)
-    qk = rope(F.rms_norm(qk, (c.head_dim,), None, c.eps) * self.qk_norm, cos, sin)
-    q, k = qk[:c.q_heads], qk[c.q_heads:]
-    k_cache.index_copy_(1, pos, k[:, None, :])
-    v_cache.index_copy_(1, pos, v)
-    a = F.scaled_dot_product_attention(q[None, :, None, :], k_cache[None], v_cache[None],
-                                       attn_mask=visible, enable_gqa=True)
-    x, = linear_grouped(a.reshape(1, nq), [self.o_proj.weight], residuals=[x])
+    a = self.attend(qk.view(c.q_heads + c.kv_heads, c.head_dim), v, pos, rot, k_cache, v_cache)
+    x, = linear_grouped(a, [self.o_proj.weight], residuals=[x])
     gate, up = linear_grouped(rms_norm(x, self.post_norm, c.eps), [self.gate_proj.weight, self.up_proj.weight])
     x, = linear_grouped(up, [self.down_proj.weight], input_gate=gate, residuals=[x])
     return x
@@ -125,13 +141,6 @@ def fuse_neighbours(model) -> int:
         blk.fused = bool(ok)
         n += int(ok)
     return n
-
-
-def rope(x, cos, sin):
-    """x [heads, d] (bf16), cos/sin [1, d/2] (fp32): rotate-half convention."""
-    half = x.shape[-1] // 2
-    x1, x2 = x[..., :half].float(), x[..., half:].float()
-    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), -1).to(x.dtype)
 
 
 def greedy(logits):
@@ -161,7 +170,13 @@ class Decoder(nn.Module):
         c = self.c
         inv = 1.0 / (c.rope_theta ** (torch.arange(0, c.head_dim, 2, device=device).float() / c.head_dim))
         ang = torch.arange(c.max_len, device=device).float()[:, None] * inv[None, :]
-        self.cos, self.sin = ang.cos(), ang.sin()                        # [max_len, d/2]
+        # per position: cosines twice, sines with the sign of the rotate-half convention
+        # (out = x * cos + swap_halves(x) * sin), one row per head with the softmax scale in the q rows
+        cos, sin = torch.cat((ang.cos(), ang.cos()), -1), torch.cat((-ang.sin(), ang.sin()), -1)      # [max_len, d]
+        scale = torch.ones(c.q_heads + c.kv_heads, 1, device=device)
+        scale[:c.q_heads] = c.head_dim ** -0.5
+        self.head_scale = scale
+        self.cos, self.sin = cos, sin
         self.k_cache = torch.zeros(c.layers, c.kv_heads, c.max_len, c.head_dim, dtype=torch.bfloat16, device=device)
         self.v_cache = torch.zeros_like(self.k_cache)
         self.slots = torch.arange(c.max_len, device=device)
@@ -174,10 +189,10 @@ class Decoder(nn.Module):
         and ``out[pos]``, advances ``pos``.  Device tensors only."""
         pos = self.pos
         x = self.embed(self.token.clamp(0, self.c.vocab - 1))            # [1, hidden]
-        cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
-        visible = (self.slots <= pos).view(1, 1, 1, -1)
+        rot = (self.cos.index_select(0, pos) * self.head_scale, self.sin.index_select(0, pos) * self.head_scale,
+               torch.where(self.slots <= pos, 0.0, float("-inf")).view(1, 1, -1), self.cos, self.sin)
         for i, blk in enumerate(self.blocks):
-            x = blk(x, pos, cos, sin, visible, self.k_cache[i], self.v_cache[i])
+            x = blk(x, pos, rot, self.k_cache[i], self.v_cache[i])
         logits = self.lm_head(rms_norm(x, self.norm, self.c.eps))
         nxt = greedy(logits)
         self.out.index_copy_(0, pos, nxt)
@@ -274,6 +289,9 @@ def parse_args(argv=None):
     ap.add_argument("--small", action="store_true", help="tiny shapes (smoke run)")
     ap.add_argument("--no-group", action="store_true", help="q/k/v and gate/up as separate launches")
     ap.add_argument("--no-fuse", action="store_true", help="norms, silu*mul and residual additions as separate PyTorch kernels")
+    ap.add_argument("--torch-attention", action="store_true",
+                    help="norm, rotation, cache update and attention of a layer as torch operations (14 kernels) instead "
+                         "of the library's one launch")
     ap.add_argument("--profile", action="store_true",
                     help="only the compressed model as it is served (grouped, fused), one run of --tokens tokens, no raw "
                          "model and no logit comparison: the run to put under rocprofv3 --kernel-trace")
@@ -291,6 +309,7 @@ def run(args) -> dict:
     c = Config(layers=args.layers)
     if args.small:
         c = Config(layers=2, hidden=512, intermediate=1024, q_heads=4, kv_heads=2, head_dim=128, vocab=4096)
+    Block.kernel_attention = not args.torch_attention
     model = build(c, device)
     g = torch.Generator().manual_seed(1)
     prompt = torch.randint(0, c.vocab, (args.prompt,), generator=g)
@@ -379,6 +398,8 @@ def run(args) -> dict:
                     f"{c.q_heads}/{c.kv_heads} heads, vocab {c.vocab}), random init N(0,0.02), bs=1, "
                     f"{args.prompt}-token prompt, {args.tokens} greedy tokens, static KV {c.max_len}, hipGraph step",
         "algo": args.algo, "modules": kinds,
+        "attention": ("torch operations: 14 kernels per layer" if args.torch_attention else
+                      "one launch per layer (RMSNorm and rotation of q/k, cache update, softmax(qk)v), raw and compressed alike"),
         "raw_tokens_per_s": round(args.tokens / raw_s, 2), "compressed_tokens_per_s": round(args.tokens / new_s, 2),
         "compressed_over_raw": round(raw_s / new_s, 4),
         "launches": ("q/k/v and gate/up one launch each" if single_s is not None else "one launch per linear")

@@ -26,6 +26,7 @@ _SIGNATURES = {
     "bhi_chunks_per_group": (_i32, [_i32, _i32, _i32]),
     "bhi_last_error_string": (ctypes.c_char_p, []),
     "bhi_stream_read": (_i64, [_vp, _i64, _i32, _i32, _vp, _vp]),
+    "bhi_decode_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, ctypes.c_float, ctypes.c_float, _vp]),
     "bhi_gemv_bf16_huffman": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,
                                      _i32, _i32, _i32, _i32, _vp]),
     "bhi_huffman_decode": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp,

@@ -1,4 +1,5 @@
-// Fused decode + matrix product for 9..32 rows of X: the weights go from the decoder's
+// Fused decode + matrix product for up to 32 rows of X (the path for 9..32 rows, and from 3 rows on
+// large layers): the weights go from the decoder's
 // registers straight into matrix-core instructions, the compressed bytes are read once
 // and no BF16 weight ever reaches HBM.
 //
@@ -15,19 +16,23 @@
 // quad q, the sums of rows 0..3 for batch 4q+j over column block b (4 registers per quad).
 //
 // X does not come from global memory per wavefront (at 32 rows that would be 8 KB per
-// wavefront and step against 0.7 KB of weights): the block's wavefronts walk the same
-// columns in lockstep, one window of four steps at a time, and the window's slice of X is
-// staged in LDS once per block in the exact order the lanes read it (conflict free,
-// 16 bytes per lane and instruction), double buffered, one barrier per window (a barrier that
-// orders LDS only: the global loads of the next window stay in flight across it).
+// wavefront and step against 0.7 KB of weights): the block's wavefronts (8, 12 or 16 of them)
+// walk the same columns in lockstep, one window of four steps at a time, and the window's
+// slice of X is staged in LDS once per block in the exact order the lanes read it (conflict
+// free, 16 bytes per lane and instruction), double buffered, one barrier per window (a barrier
+// that orders LDS only: the global loads of the next window stay in flight across it).
 //
 // Measured on MI355X, Student-t weights, rotating over 640 MB of clones: 12288x4096 at 16 / 32
-// rows 29.8 / 40.7 us against 56 us for decode-to-BF16 + library GEMM; 4096x12288 (6 K slices)
-// 43 / 61 us against 54-56 us.  Taking the X reads out (wrong results) saves 1.6 / 3.8 us, the
-// barriers 2.8 / 5.7 us; requesting rem bytes, rows and X two windows ahead instead of one was
-// slower (31.7-35.5 us: 128 registers, and nothing was waiting for those loads).  What is left
-// is the decode itself at three to four wavefronts per SIMD -- LDS (two windows of X, rings,
-// table) and 100-128 registers allow no more -- against six in the GEMV.
+// rows 25.0 / 32.2 us against 56 us for decode-to-BF16 + library GEMM; 4096x12288 (2 / 3 K
+// slices) 32 / 45 us against 54-56 us.  Taking the X reads out (wrong results) saves 1.6 / 3.8 us,
+// the barriers 2.8 / 5.7 us; requesting rem bytes, rows and X two windows ahead instead of one
+// was slower (128 registers, and nothing was waiting for those loads).  A compute unit gets
+// through 1.5 times the row groups with 16 resident wavefronts that it does with 8, and no more
+// with 24: the lockstep makes a block as slow as its slowest wavefront in every window, so what
+// counts is that the grid covers the 256 units evenly (mma_plan below).  From 3 to 8 rows the
+// kernel also beats the GEMV on large layers (37888x3584 at 4 rows 39.8 against 44.4 us, at 8
+// rows 45.0 against 58.7 us): one load of X per block instead of one per wavefront, two matrix
+// instructions per batch quad and step instead of four dot products per batch row.
 //
 // Few row groups (M < 8192) would leave most of the GPU idle, so the tasks of a row group
 // can be dealt to up to 8 blocks (K slices).  Their partial sums meet in a workspace in

@@ -7,7 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
-SOURCES = ["bhi_api.hip", "bhi_huffman.hip", "bhi_ans.hip", "bhi_nibble.hip", "bhi_reference.hip"]
+SOURCES = ["bhi_api.hip", "bhi_huffman.hip", "bhi_ans.hip", "bhi_nibble.hip", "bhi_reference.hip", "bhi_attention.hip"]
 LIB = os.path.join(PKG, "libbhi_hip.so")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

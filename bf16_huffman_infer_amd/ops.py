@@ -382,6 +382,45 @@ def silu_mul(gate: Tensor, up: Tensor) -> Tensor:
     return out
 
 
+def decode_attention(qk: Tensor, v: Tensor, norm_weight, cos: Tensor, sin: Tensor, pos: Tensor, k_cache: Tensor,
+                     v_cache: Tensor, out: Tensor = None, eps: float = 1e-6, scale: float = None) -> Tensor:
+    """The attention step of one new token of a decoder layer in one launch (no counterpart in the
+    reference, which leaves attention to the model code): per-head RMSNorm (times ``norm_weight``,
+    bf16 ``[q_heads + kv_heads, 128]`` or None) and rotation of the projected heads ``qk`` (bf16
+    ``[q_heads + kv_heads, 128]``, q heads first) by row ``pos`` of ``cos`` / ``sin`` (fp32
+    ``[max_len, 128]``, ``out = x * cos + swap_halves(x) * sin``), ``k`` and ``v`` (bf16 ``[kv_heads, 128]``)
+    written into slot ``pos`` of ``k_cache`` / ``v_cache`` (bf16 ``[kv_heads, max_len, 128]``), and
+    ``softmax(q k^T * scale) v`` over slots ``0..pos`` per q head.  ``pos`` is an int64 tensor of one
+    element ON THE DEVICE: a recorded graph reads it at every replay.  Returns ``out`` (bf16
+    ``[q_heads, 128]``)."""
+    heads, d = qk.shape
+    kv_heads, max_len, _ = k_cache.shape
+    q_heads = heads - kv_heads
+    if tuple(v.shape) != (kv_heads, d) or tuple(v_cache.shape) != (kv_heads, max_len, d):
+        raise RuntimeError("v must be [kv_heads, head_dim] and the caches [kv_heads, max_len, head_dim]")
+    if tuple(cos.shape) != (max_len, d) or tuple(sin.shape) != (max_len, d):
+        raise RuntimeError(f"cos and sin must be [{max_len}, {d}]")
+    if pos.numel() != 1 or pos.dtype != torch.int64 or pos.device != qk.device:
+        raise RuntimeError("pos must be one int64 on the device of qk")
+    if norm_weight is not None and tuple(norm_weight.shape) != (heads, d):
+        raise RuntimeError(f"norm_weight must be [{heads}, {d}]")
+    if out is None:
+        out = torch.empty((q_heads, d), dtype=torch.bfloat16, device=qk.device)
+    elif tuple(out.shape) != (q_heads, d):
+        raise RuntimeError(f"out must be [{q_heads}, {d}]")
+    lib = _lib.load()
+    with torch.cuda.device(qk.device):
+        rc = lib.bhi_decode_attention(
+            _req(qk, torch.bfloat16, "qk"), _req(v, torch.bfloat16, "v", qk),
+            None if norm_weight is None else _req(norm_weight, torch.bfloat16, "norm_weight", qk),
+            _req(cos, torch.float32, "cos", qk), _req(sin, torch.float32, "sin", qk), pos.data_ptr(),
+            _req(k_cache, torch.bfloat16, "k_cache", qk), _req(v_cache, torch.bfloat16, "v_cache", qk),
+            _req(out, torch.bfloat16, "out", qk), q_heads, kv_heads, d, max_len, float(eps),
+            float(d ** -0.5 if scale is None else scale), _stream(qk))
+    _lib.check(rc, "decode_attention")
+    return out
+
+
 def _fill_member(m, w, Y: Tensor, bias, ref: Tensor) -> bool:
     """Fills one ``bhi_gemv_member`` from a weight module; returns whether it is a Huffman weight."""
     huffman = hasattr(w, "LUT1")

@@ -247,6 +247,23 @@ int bhi_reference_ans_decode(const void* A_rem, const void* A_exp, int64_t exp_w
                              void* Y, const void* offsets, const void* LUT,
                              int split_k, int M, int Ks, void* stream);
 
+/* No counterpart in the reference (which leaves attention to the model code around its linear
+ * layers): the attention step of ONE new token of a decoder layer in one launch, so that a
+ * recorded decode step is not dominated by small kernels between this library's launches.
+ * Per head: RMSNorm of the projected q and k heads (fp32, then times `norm_weight` -- bf16
+ * [q_heads + kv_heads, head_dim], or NULL), rotation by the angles of the token's position
+ * (`cos`, `sin`: fp32 [max_len, head_dim]; out = x * cos + swap_halves(x) * sin, so `sin` holds
+ * -sin in its first half and +sin in its second), k and v written to slot `*pos` of the caches
+ * (bf16 [kv_heads, max_len, head_dim]), then softmax(q . k * scale) over slots 0 .. *pos times v
+ * for each q head (q heads h * q_heads / kv_heads .. share k/v head h), `out` bf16
+ * [q_heads, head_dim].  `qk` is bf16 [q_heads + kv_heads, head_dim] (q heads first), `v` bf16
+ * [kv_heads, head_dim]; `pos` points to one int64 in DEVICE memory (a recorded graph follows
+ * it); head_dim must be 128, max_len at most 8192.  q, k, the softmax weights and the output
+ * are rounded to BF16 where a chain of BF16 torch operations would round them. */
+int bhi_decode_attention(const void* qk, const void* v, const void* norm_weight, const void* cos, const void* sin,
+                         const void* pos, void* k_cache, void* v_cache, void* out, int q_heads, int kv_heads,
+                         int head_dim, int max_len, float eps, float scale, void* stream);
+
 /* No counterpart in the reference: a measurement helper.  Enqueues a kernel in which
  * `wavefronts` wavefronts (a positive multiple of 4) each load a contiguous span of `src`
  * (four 16-byte loads in flight per lane, with or without the non-temporal hint) and keep

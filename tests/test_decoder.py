@@ -38,7 +38,12 @@ def test_decoder_matches_transformers_qwen3():
             got.append(m.step()[0].clone())
     got = torch.stack(got)
     torch.testing.assert_close(got.float(), ref.float(), rtol=0, atol=0.05)
-    assert torch.equal(got.argmax(-1), ref.argmax(-1))
+    # the same token wherever the reference's best logit leads its second best by more than the noise
+    # (q and k stay in fp32 from the RMSNorm to the end of the rotation here, transformers rounds in between)
+    top = ref.float().topk(2, -1).values
+    clear = (top[:, 0] - top[:, 1]) > 0.1
+    assert clear.any()
+    assert torch.equal(got.argmax(-1)[clear], ref.argmax(-1)[clear])
 
 
 @pytest.mark.gpu
