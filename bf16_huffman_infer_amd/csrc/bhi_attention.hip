@@ -118,9 +118,16 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
     }
     __syncthreads();
 
-    // ---- scores of the slots before the token's own (those are in the cache already)
+    // ---- scores: the token's own slot from LDS (wavefront 3, two elements per lane), the slots
+    // before it from the cache
     const int rounds = (n + kAttnThreads - 1) / kAttnThreads;
     float best = -INFINITY;
+    if (wave == 3) {
+        const float own = wave_sum(__uint_as_float((uint32_t)k_new[lane] << 16) * q[lane] +
+                                   __uint_as_float((uint32_t)k_new[lane + 64] << 16) * q[lane + 64]);
+        if (lane == 0) weights[n - 1] = own;
+        best = own;
+    }
     for (int r0 = 0; r0 < rounds; r0 += 4) {
         float s[4] = {0.f, 0.f, 0.f, 0.f};
         const uint4* rows[4];
@@ -143,13 +150,8 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int j = (r0 + u) * kAttnThreads + tid;
-            if (r0 + u < rounds) {
-                float v = -INFINITY;
-                if (j < n - 1) v = s[u];
-                if (j == n - 1) {                        // the token's own slot: k from LDS
-                    v = 0.f;
-                    for (int d = 0; d < kAttnDim; ++d) v += __uint_as_float((uint32_t)k_new[d] << 16) * q[d];
-                }
+            if (r0 + u < rounds && j != n - 1) {
+                const float v = j < n - 1 ? s[u] : -INFINITY;
                 weights[j] = v;
                 best = fmaxf(best, v);
             }

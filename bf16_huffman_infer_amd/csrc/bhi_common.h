@@ -14,7 +14,7 @@
 
 namespace bhi {
 
-constexpr int kFormatVersion = 1;
+constexpr int kFormatVersion = 2;
 constexpr int kLanes = 64;
 constexpr int kGroupRows = 4;
 constexpr int kLaneCols = 8;
@@ -44,6 +44,13 @@ __host__ __device__ inline int chunks_per_group(int M, int Ks, int split_k) {
     int nc = 1;
     while (nc < kMaxChunks && (long long)(M / kGroupRows) * split_k * nc * 2 <= kTargetTasks &&
            steps / (nc * 2) >= kMinChunkSteps)
+        nc *= 2;
+    // The tasks of a row group are dealt to the four wavefronts of a block: six tasks would give
+    // two wavefronts two tasks and two of them one (4096x12288 with three splits: 32 steps on the
+    // longest wavefront where 24 would do), so a count above four that is no multiple of four
+    // is doubled once more.
+    if (split_k * nc > kWavesPerBlock && (split_k * nc) % kWavesPerBlock != 0 && nc < kMaxChunks &&
+        steps / (nc * 2) >= kMinChunkSteps)
         nc *= 2;
     return nc;
 }

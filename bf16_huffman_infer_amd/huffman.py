@@ -173,7 +173,7 @@ class LUTHuffmanEncoder:
         assert filled.all() and code == (1 << prev_len), "code is not complete"
 
         self.code_lengths[:] = 0
-        self.code_lengths[0] = 1                      # format version
+        self.code_lengths[0] = 2                      # format version
         self.code_lengths[1] = TABLE_BITS
         self.code_lengths[2] = int(self.enc_table[ESC_INDEX]) >> 16
         self.code_lengths[3] = 1 if int(counts.sum() - counts[coded].sum()) > 0 else 0   # escapes occur

@@ -70,6 +70,10 @@ def chunks_per_group(M: int, Ks: int, split_k: int) -> int:
     while (nc < MAX_CHUNKS and (M // GROUP_ROWS) * split_k * nc * 2 <= TARGET_TASKS
            and steps // (nc * 2) >= MIN_CHUNK_STEPS):
         nc *= 2
+    # a row group's tasks are dealt to four wavefronts: a count above four that is no multiple of
+    # four would leave them with unequal shares, so it is doubled once more
+    if split_k * nc > 4 and (split_k * nc) % 4 != 0 and nc < MAX_CHUNKS and steps // (nc * 2) >= MIN_CHUNK_STEPS:
+        nc *= 2
     return nc
 
 

@@ -14,7 +14,7 @@ def _task_offsets(split_k, M, words_per_task=64):
     return off.view(split_k, M), split_k * (M // 4) * words_per_task + 2048
 
 
-def _huffman_weight(M, K, header=(1, 11, 11, 0)):
+def _huffman_weight(M, K, header=(2, 11, 11, 0)):
     offsets, words = _task_offsets(1, M)
     code_lengths = torch.zeros(256, dtype=torch.uint8)
     code_lengths[:4] = torch.tensor(header, dtype=torch.uint8)
@@ -213,7 +213,7 @@ def test_workspace_of_the_fused_product_follows_the_slice_choice():
         return (need - 1024) // (rows * M * 4)
 
     assert slices(1, 12288, 4096, 16) == 1 and slices(1, 12288, 4096, 32) == 1      # 3072 row groups: never cut
-    assert slices(3, 4096, 4096, 16) == 2 and slices(3, 4096, 4096, 32) == 3        # 4096x12288, 6 tasks per group
+    assert slices(3, 4096, 4096, 16) == 4 and slices(3, 4096, 4096, 32) == 4        # 4096x12288, 12 tasks per group
     assert slices(4, 3584, 4736, 16) == 4 and slices(4, 3584, 4736, 32) == 4        # 3584x18944, 4 long tasks
     assert slices(1, 4096, 4096, 16) == 2 and slices(1, 4608, 3584, 16) == 2
     # every choice divides the tasks of a row group, and the built-in workspace holds whatever
