@@ -16,8 +16,8 @@
 //     The group's first block writes k and v into the cache; every block takes the new
 //     token's k and v from LDS / the input, so no block waits for another.
 //  2. Scores: thread t owns cache slots t, t + 256, ...; a slot's k row is 256 contiguous
-//     bytes, read 16 bytes at a time against q from LDS (broadcast reads).  Four slots are in
-//     flight per thread.
+//     bytes, requested whole (sixteen 16-byte loads in flight) and multiplied with q from LDS
+//     (broadcast reads).
 //  3. Softmax over the block (fp32; maximum and sum through wavefront reductions and LDS),
 //     the weights rounded to BF16 as a BF16 matrix product would take them.
 //  4. Output: wavefront w sums slots w, w + 4, ...; lane l owns elements 2l and 2l + 1 of the
@@ -128,33 +128,24 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
         if (lane == 0) weights[n - 1] = own;
         best = own;
     }
-    for (int r0 = 0; r0 < rounds; r0 += 4) {
-        float s[4] = {0.f, 0.f, 0.f, 0.f};
-        const uint4* rows[4];
+    for (int r = 0; r < rounds; ++r) {
+        // one slot per thread and round, its whole row requested at once (16 loads in flight)
+        const int j = r * kAttnThreads + tid;
+        const uint4* row = (const uint4*)(kc + (size_t)(j < n - 1 ? j : 0) * kAttnDim);   // past the end: any valid row, dropped below
+        uint4 kk[kAttnDim / 8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            int j = (r0 + u) * kAttnThreads + tid;
-            j = j < n - 1 ? j : 0;                      // past the end: any valid row, the result is dropped
-            rows[u] = (const uint4*)(kc + (size_t)j * kAttnDim);
-        }
-#pragma unroll 4
+        for (int c = 0; c < kAttnDim / 8; ++c) kk[c] = row[c];
+        float s = 0.f;
+#pragma unroll
         for (int c = 0; c < kAttnDim / 8; ++c) {
             const float4 q0 = *(const float4*)(q + 8 * c), q1 = *(const float4*)(q + 8 * c + 4);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint4 kk = rows[u][c];
-                s[u] += bf16_lo(kk.x) * q0.x + bf16_hi(kk.x) * q0.y + bf16_lo(kk.y) * q0.z + bf16_hi(kk.y) * q0.w
-                      + bf16_lo(kk.z) * q1.x + bf16_hi(kk.z) * q1.y + bf16_lo(kk.w) * q1.z + bf16_hi(kk.w) * q1.w;
-            }
+            s += bf16_lo(kk[c].x) * q0.x + bf16_hi(kk[c].x) * q0.y + bf16_lo(kk[c].y) * q0.z + bf16_hi(kk[c].y) * q0.w
+               + bf16_lo(kk[c].z) * q1.x + bf16_hi(kk[c].z) * q1.y + bf16_lo(kk[c].w) * q1.z + bf16_hi(kk[c].w) * q1.w;
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int j = (r0 + u) * kAttnThreads + tid;
-            if (r0 + u < rounds && j != n - 1) {
-                const float v = j < n - 1 ? s[u] : -INFINITY;
-                weights[j] = v;
-                best = fmaxf(best, v);
-            }
+        if (j != n - 1) {
+            const float v = j < n - 1 ? s : -INFINITY;
+            weights[j] = v;
+            best = fmaxf(best, v);
         }
     }
     best = wave_max(best);
@@ -177,18 +168,26 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
     float o0 = 0.f, o1 = 0.f;
     const uint32_t* vrow = (const uint32_t*)vc + lane;
     int j = wave;
+    for (; j + 60 < n - 1; j += 64) {                   // sixteen rows in flight per wavefront
+        uint32_t x[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) x[u] = vrow[(size_t)(j + 4 * u) * (kAttnDim / 2)];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const float w = __uint_as_float((uint32_t)f32_to_bf16_rne(weights[j + 4 * u] * inv) << 16);
+            o0 += w * bf16_lo(x[u]);
+            o1 += w * bf16_hi(x[u]);
+        }
+    }
     for (; j + 12 < n - 1; j += 16) {
         uint32_t x[4];
-        float w[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x[u] = vrow[(size_t)(j + 4 * u) * (kAttnDim / 2)];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            x[u] = vrow[(size_t)(j + 4 * u) * (kAttnDim / 2)];
-            w[u] = __uint_as_float((uint32_t)f32_to_bf16_rne(weights[j + 4 * u] * inv) << 16);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            o0 += w[u] * bf16_lo(x[u]);
-            o1 += w[u] * bf16_hi(x[u]);
+            const float w = __uint_as_float((uint32_t)f32_to_bf16_rne(weights[j + 4 * u] * inv) << 16);
+            o0 += w * bf16_lo(x[u]);
+            o1 += w * bf16_hi(x[u]);
         }
     }
     for (; j < n - 1; j += 4) {
