@@ -349,7 +349,7 @@ struct DotPolicy {
     struct Slot { uint2 rem; uint4 x; uint4 a; };            // x: the lane's X pair of batch rows 0..3; a: gamma or gate pairs
     struct Piped { uint4 x, a; int i, t; };
     const uint2* rem0;
-    const uint2* spare_rem;  // kSegLong * 512 readable bytes that are cache resident (the decode table, or the task's start)
+    const uint2* spare_rem;  // kSegLong * 512 readable bytes that are cache resident (the decode table, the offsets, or the task's start)
     const uint32_t* xq0;     // this lane's X pair of batch row 0, first step of the task
     const uint32_t* aq0;     // the same position in gamma (kXRms) or in gate row 0 (kXSiluMul)
     float rs[BS <= 4 ? BS : 1];   // kXRms: the rows' scales
@@ -636,7 +636,12 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
             pol.aq0 = XM == kXPlain ? nullptr
                                     : (const uint32_t*)(grp.xaux + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
-            pol.spare_rem = Codec::kTableWords * 4 >= kSegLong * kLanes * 8 ? (const uint2*)table + lane : pol.rem0;
+            // loads nobody needs go to bytes that are in cache anyway: the decode table where it is
+            // long enough, else the offsets array (rounded up to an 8-byte boundary), else the task's start
+            constexpr int kSpareBytes = kSegLong * kLanes * 8;
+            if (Codec::kTableWords * 4 >= kSpareBytes) pol.spare_rem = (const uint2*)table + lane;
+            else if ((long long)s.M * s.split_k * 4 >= kSpareBytes + 8) pol.spare_rem = (const uint2*)(((uintptr_t)offsets + 7) & ~(uintptr_t)7) + lane;
+            else pol.spare_rem = pol.rem0;
             // looked at only now: the flag's load has been in flight together with the offsets'
             const bool variant = Codec::variant_test(pin_uniform(variant_word), header);
             if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
