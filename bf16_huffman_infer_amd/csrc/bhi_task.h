@@ -349,7 +349,7 @@ struct DotPolicy {
     struct Slot { uint2 rem; uint4 x; uint4 a; };            // x: the lane's X pair of batch rows 0..3; a: gamma or gate pairs
     struct Piped { uint4 x, a; int i, t; };
     const uint2* rem0;
-    const uint2* spare_rem;  // kSegLong * 512 readable bytes that are cache resident (the decode table, the offsets, or the task's start)
+    const uint2* spare_rem;  // kSegLong * 512 readable bytes that are cache resident (the decode table, or the start of the task's exponent stream)
     const uint32_t* xq0;     // this lane's X pair of batch row 0, first step of the task
     const uint32_t* aq0;     // the same position in gamma (kXRms) or in gate row 0 (kXSiluMul)
     float rs[BS <= 4 ? BS : 1];   // kXRms: the rows' scales
@@ -630,18 +630,21 @@ void gemv_kernel(const uint16_t* __restrict__ X, int first1, int first2, int fir
         for (int kc = p; kc < per_group; kc += P) {
             const TaskId id = task_of(s, kc);
             typename Codec::Cursor cur;
-            cur.open(A_exp, task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words), lane, rings[wave]);
+            const TaskSpan span = task_span(offsets, s.M, s.split_k, s.nc, id.k, g, id.c, s.total_words);
+            cur.open(A_exp, span, lane, rings[wave]);
             pol.rem0 = (const uint2*)(A_rem + ((size_t)id.k * s.M + (size_t)kGroupRows * g) * s.Ks) + (size_t)id.t0 * kLanes + lane;
             pol.xq0 = (const uint32_t*)(X + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.aq0 = XM == kXPlain ? nullptr
                                     : (const uint32_t*)(grp.xaux + (size_t)id.k * s.Ks + (size_t)id.t0 * kStepCols) + lane;
             pol.last = id.t1 - id.t0 - 1;
             // loads nobody needs go to bytes that are in cache anyway: the decode table where it is
-            // long enough, else the offsets array (rounded up to an 8-byte boundary), else the task's start
-            constexpr int kSpareBytes = kSegLong * kLanes * 8;
-            if (Codec::kTableWords * 4 >= kSpareBytes) pol.spare_rem = (const uint2*)table + lane;
-            else if ((long long)s.M * s.split_k * 4 >= kSpareBytes + 8) pol.spare_rem = (const uint2*)(((uintptr_t)offsets + 7) & ~(uintptr_t)7) + lane;
-            else pol.spare_rem = pol.rem0;
+            // long enough, else the start of the task's own exponent stream (read moments ago; the
+            // zero tail behind the last stream keeps kSegLong * 512 bytes readable from any task's
+            // start).  One region for every wavefront -- the offsets array was tried -- makes a few
+            // cache lines hot and costs 4 % on the rANS block step.
+            static_assert(kTailPadWords * 4 >= kSegLong * kLanes * 8, "the tail pad covers a segment's spare loads");
+            if (Codec::kTableWords * 4 >= kSegLong * kLanes * 8) pol.spare_rem = (const uint2*)table + lane;
+            else pol.spare_rem = (const uint2*)(A_exp + (span.base & ~1u)) + lane;
             // looked at only now: the flag's load has been in flight together with the offsets'
             const bool variant = Codec::variant_test(pin_uniform(variant_word), header);
             if (variant) run_task<true, S>(cur, lut, pol, id.t1 - id.t0, stage_all);
