@@ -92,6 +92,23 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
     const float *cs = a.cos + (size_t)p * kAttnDim, *sn = a.sin + (size_t)p * kAttnDim;
     const bool writer = h % group == 0;
 
+    // What depends on the position only is requested now, ahead of the q/k work and its barrier:
+    // the k row of this thread's first slot and the v rows of the wavefront's first sixteen slots
+    // (clamped to a valid row where there is no such slot; those values are never used).
+    uint4 kk[kAttnDim / 8];
+    {
+        const uint4* row = (const uint4*)(kc + (size_t)(tid < n - 1 ? tid : 0) * kAttnDim);
+#pragma unroll
+        for (int c = 0; c < kAttnDim / 8; ++c) kk[c] = row[c];
+    }
+    const uint32_t* vrow = (const uint32_t*)vc + lane;
+    uint32_t v_first[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const int j = wave + 4 * u;
+        v_first[u] = vrow[(size_t)(j < n - 1 ? j : 0) * (kAttnDim / 2)];
+    }
+
     if (wave == 0) {
         const float2 r = norm_rotate(a.qk + (size_t)h * kAttnDim, a.norm_w ? a.norm_w + (size_t)h * kAttnDim : nullptr,
                                      cs, sn, lane, a.eps, a.scale);
@@ -131,10 +148,11 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
     for (int r = 0; r < rounds; ++r) {
         // one slot per thread and round, its whole row requested at once (16 loads in flight)
         const int j = r * kAttnThreads + tid;
-        const uint4* row = (const uint4*)(kc + (size_t)(j < n - 1 ? j : 0) * kAttnDim);   // past the end: any valid row, dropped below
-        uint4 kk[kAttnDim / 8];
+        if (r > 0) {
+            const uint4* row = (const uint4*)(kc + (size_t)(j < n - 1 ? j : 0) * kAttnDim);   // past the end: any valid row, dropped below
 #pragma unroll
-        for (int c = 0; c < kAttnDim / 8; ++c) kk[c] = row[c];
+            for (int c = 0; c < kAttnDim / 8; ++c) kk[c] = row[c];
+        }
         float s = 0.f;
 #pragma unroll
         for (int c = 0; c < kAttnDim / 8; ++c) {
@@ -166,8 +184,16 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(const At
 
     // ---- weighted sum of the v rows: wavefront w takes slots w, w + 4, ...
     float o0 = 0.f, o1 = 0.f;
-    const uint32_t* vrow = (const uint32_t*)vc + lane;
-    int j = wave;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {                      // the rows requested at the start
+        const int j = wave + 4 * u;
+        if (j < n - 1) {
+            const float w = __uint_as_float((uint32_t)f32_to_bf16_rne(weights[j] * inv) << 16);
+            o0 += w * bf16_lo(v_first[u]);
+            o1 += w * bf16_hi(v_first[u]);
+        }
+    }
+    int j = wave + 64;
     for (; j + 60 < n - 1; j += 64) {                   // sixteen rows in flight per wavefront
         uint32_t x[16];
 #pragma unroll
